@@ -1,0 +1,128 @@
+/*
+ * fp8gemm.h -- C ABI of the MI355X (gfx950) FP8 GEMM library.
+ *
+ * Every entry point computes, on the current HIP device,
+ *
+ *     out[i*n + j] = sum_{t<k} float(a[i*k + t]) * float(b[j*k + t])
+ *
+ * with A row-major m x k, B stored n x k ("row-col"), C row-major m x n fp32,
+ * fp32 accumulation, pure overwrite (C is never read; no alpha/beta/scales).
+ * a, b, out are caller-owned DEVICE pointers that must not alias.  Launches
+ * are asynchronous on the given HIP stream (NULL = the default stream).
+ * Return value: a hipError_t as int, 0 (hipSuccess) on success,
+ * 1 (hipErrorInvalidValue) for null pointers, non-positive dimensions, bad
+ * format / stage / algorithm codes.  Any m, k, n >= 1 is computed in full
+ * (the reference silently leaves tiles past the last multiple of 128 unwritten,
+ * GEMM/src/gemm.cu:45-47; this library does not).
+ *
+ * Format codes: 0 = OCP E4M3 (bias 7, max 448, no Inf), 1 = OCP E5M2.
+ */
+#ifndef FP8GEMM_H
+#define FP8GEMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FP8GEMM_E4M3 0
+#define FP8GEMM_E5M2 1
+
+/* Kernel families, for fp8gemm_launch_algo (testing / tuning hook). */
+#define FP8GEMM_ALGO_AUTO 0    /* shape-based choice, what every other entry uses */
+#define FP8GEMM_ALGO_DIRECT 1  /* one wave per 32x32 tile, global->register, any shape */
+#define FP8GEMM_ALGO_TILE 2    /* LDS-tiled MFMA kernel for compute-bound shapes */
+#define FP8GEMM_ALGO_SKINNY 3  /* B-streaming kernel for small m (HBM-bound) */
+
+/*
+ * The eight per-precision launch entry points.  Each replaces one C++ overload
+ * of the reference's launch API (GEMM/include/gemm.cuh), argument order
+ * (m, k, n, a, b, out) as there, default stream as there
+ * (GEMM/src/gemm.cu:263-285).  "stage2" backs gemm::GEMM, "stage4" backs
+ * gemm::GEMM4; the stage count selects the LDS pipeline depth of the tiled
+ * kernel and never changes the result's contract.
+ */
+int fp8gemm_e4m3_e4m3_stage2(int m, int k, int n, const void *a, const void *b, float *out); /* gemm.cuh:12-15 */
+int fp8gemm_e4m3_e4m3_stage4(int m, int k, int n, const void *a, const void *b, float *out); /* gemm.cuh:18-21 */
+int fp8gemm_e5m2_e5m2_stage2(int m, int k, int n, const void *a, const void *b, float *out); /* gemm.cuh:24-27 */
+int fp8gemm_e5m2_e5m2_stage4(int m, int k, int n, const void *a, const void *b, float *out); /* gemm.cuh:30-33 */
+int fp8gemm_e4m3_e5m2_stage2(int m, int k, int n, const void *a, const void *b, float *out); /* gemm.cuh:36-39 */
+int fp8gemm_e4m3_e5m2_stage4(int m, int k, int n, const void *a, const void *b, float *out); /* gemm.cuh:41-44 */
+int fp8gemm_e5m2_e4m3_stage2(int m, int k, int n, const void *a, const void *b, float *out); /* gemm.cuh:47-50 */
+int fp8gemm_e5m2_e4m3_stage4(int m, int k, int n, const void *a, const void *b, float *out); /* gemm.cuh:52-55 */
+
+/*
+ * Generic form of the above (the launchers GEMMex / GEMMex4 of
+ * GEMM/src/gemm.cu:263-277, 670-686 folded into one): formats and stage count
+ * as arguments, explicit stream (a hipStream_t passed as void*).
+ * stages must be 2 or 4.
+ */
+int fp8gemm_launch(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
+                   float *out, int stages, void *stream);
+
+/* As fp8gemm_launch, but forces one kernel family (FP8GEMM_ALGO_*).  Returns
+ * hipErrorInvalidValue when the family cannot run the shape. */
+int fp8gemm_launch_algo(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
+                        float *out, int stages, int algo, void *stream);
+
+/*
+ * Tuning hook with no counterpart in the reference: forces a kernel family
+ * and one of its compiled shape variants (0 .. fp8gemm_num_variants(algo)-1,
+ * -1 = the default for the shape).  For FP8GEMM_ALGO_SKINNY, variant may add
+ * 16 * columns-per-wave/16 to override the planned column count per wave, and
+ * split_k > 0 overrides the planned split-K factor.
+ */
+int fp8gemm_launch_tuned(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
+                         float *out, int algo, int variant, int split_k, void *stream);
+int fp8gemm_num_variants(int algo);
+
+/* Which family FP8GEMM_ALGO_AUTO picks for a shape (pure host logic). */
+int fp8gemm_select_algo(int m, int k, int n);
+
+/* Bytes of device scratch the split-K path of the skinny kernel keeps cached
+ * per device for a shape (0 when the shape needs none).  The scratch is the
+ * only allocation the library ever makes; it is grown on demand, reused by
+ * later calls and shared by all streams of the device, so calls that overlap
+ * on one device and both need it must be ordered by the caller. */
+size_t fp8gemm_scratch_bytes(int m, int k, int n);
+
+/* Text for a return code (hipGetErrorString). */
+const char *fp8gemm_error_string(int code);
+
+/* Library version, major*100 + minor. */
+int fp8gemm_version(void);
+
+/*
+ * Host-side fp8 codec (bit-exact OCP conversions; the arithmetic the
+ * reference gets from the converting constructor / operator float of its fp8
+ * types, GEMM/include/bm_test_utils.h:139 and GEMM/gemm_main.cpp:48).
+ */
+uint8_t fp8gemm_encode_one(float x, int fmt);
+float fp8gemm_decode_one(uint8_t code, int fmt);
+void fp8gemm_encode(const float *src, uint8_t *dst, size_t count, int fmt);
+void fp8gemm_decode(const uint8_t *src, float *dst, size_t count, int fmt);
+
+/*
+ * Seeded synthetic matrices written straight to fp8 codes in HOST memory (the
+ * role of MakeDenseMatrix, GEMM/include/bm_test_utils.h:131-143).  All are
+ * counter-based (element i depends only on seed and i), so results do not
+ * depend on thread count.
+ *   uniform    : U(lo, hi)
+ *   normal     : mean + sigma * N(0,1)
+ *   weights    : sigma * N(0,1), then scaled so the largest magnitude maps to
+ *                the format's largest finite value (per-tensor scaling)
+ *   loguniform : +-2^u, u uniform over the format's whole finite exponent
+ *                range (subnormals included), never NaN/Inf
+ */
+void fp8gemm_fill_uniform(uint8_t *dst, size_t count, int fmt, uint64_t seed, float lo, float hi);
+void fp8gemm_fill_normal(uint8_t *dst, size_t count, int fmt, uint64_t seed, float mean, float sigma);
+void fp8gemm_fill_weights(uint8_t *dst, size_t count, int fmt, uint64_t seed, float sigma);
+void fp8gemm_fill_loguniform(uint8_t *dst, size_t count, int fmt, uint64_t seed);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* FP8GEMM_H */

@@ -1,0 +1,203 @@
+"""Python plumbing over the C ABI of the gfx950 FP8 GEMM library.
+
+The product is the shared library ``lib/libfp8gemm.so`` (HIP kernels + C ABI,
+``include/fp8gemm.h``) and the C++ harness under ``GEMM/``.  This module only
+loads the library with ctypes and passes torch device pointers through, so
+that tests and the benchmark can drive the same entry points a C++ caller
+binds.  There is no fallback: if the library is missing, loading raises.
+
+``GEMM`` / ``GEMM4`` mirror the reference's launch API
+(GEMM/include/gemm.cuh:11-55): argument order (m, k, n, a, b, out), the
+operand pairing chosen by the operand types (here: torch.float8_e4m3fn /
+torch.float8_e5m2 tensors).
+"""
+import ctypes
+import os
+import subprocess
+
+E4M3 = 0
+E5M2 = 1
+ALGO_AUTO, ALGO_DIRECT, ALGO_TILE, ALGO_SKINNY = 0, 1, 2, 3
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libfp8gemm.so")
+HARNESS_DIR = os.path.join(_HERE, "GEMM")
+HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "fp8gemm.h")
+
+_lib = None
+
+ENTRY_POINTS = [
+    "fp8gemm_e4m3_e4m3_stage2", "fp8gemm_e4m3_e4m3_stage4",
+    "fp8gemm_e5m2_e5m2_stage2", "fp8gemm_e5m2_e5m2_stage4",
+    "fp8gemm_e4m3_e5m2_stage2", "fp8gemm_e4m3_e5m2_stage4",
+    "fp8gemm_e5m2_e4m3_stage2", "fp8gemm_e5m2_e4m3_stage4",
+]
+
+
+class Fp8GemmError(RuntimeError):
+    pass
+
+
+def build(jobs=8):
+    """Compile the library and the harness for gfx950 (hipcc; no GPU needed)."""
+    subprocess.check_call(["make", "-C", HARNESS_DIR, "-j", str(jobs), "lib", "gemm"])
+
+
+def lib():
+    """The loaded C ABI.  Raises if the shared library has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise Fp8GemmError(
+            "libfp8gemm.so is not built (%s); run __graft_entry__.build() or "
+            "`make -C tensor-core-fp8_amd/GEMM lib`" % LIB_PATH)
+    L = ctypes.CDLL(LIB_PATH)
+    vp, ci = ctypes.c_void_p, ctypes.c_int
+    for name in ENTRY_POINTS:
+        fn = getattr(L, name)
+        fn.restype = ci
+        fn.argtypes = [ci, ci, ci, vp, vp, vp]
+    L.fp8gemm_launch.restype = ci
+    L.fp8gemm_launch.argtypes = [ci, ci, ci, vp, ci, vp, ci, vp, ci, vp]
+    L.fp8gemm_launch_algo.restype = ci
+    L.fp8gemm_launch_algo.argtypes = [ci, ci, ci, vp, ci, vp, ci, vp, ci, ci, vp]
+    L.fp8gemm_launch_tuned.restype = ci
+    L.fp8gemm_launch_tuned.argtypes = [ci, ci, ci, vp, ci, vp, ci, vp, ci, ci, ci, vp]
+    L.fp8gemm_num_variants.restype = ci
+    L.fp8gemm_num_variants.argtypes = [ci]
+    L.fp8gemm_select_algo.restype = ci
+    L.fp8gemm_select_algo.argtypes = [ci, ci, ci]
+    L.fp8gemm_scratch_bytes.restype = ctypes.c_size_t
+    L.fp8gemm_scratch_bytes.argtypes = [ci, ci, ci]
+    L.fp8gemm_error_string.restype = ctypes.c_char_p
+    L.fp8gemm_error_string.argtypes = [ci]
+    L.fp8gemm_version.restype = ci
+    L.fp8gemm_encode_one.restype = ctypes.c_uint8
+    L.fp8gemm_encode_one.argtypes = [ctypes.c_float, ci]
+    L.fp8gemm_decode_one.restype = ctypes.c_float
+    L.fp8gemm_decode_one.argtypes = [ctypes.c_uint8, ci]
+    L.fp8gemm_encode.restype = None
+    L.fp8gemm_encode.argtypes = [vp, vp, ctypes.c_size_t, ci]
+    L.fp8gemm_decode.restype = None
+    L.fp8gemm_decode.argtypes = [vp, vp, ctypes.c_size_t, ci]
+    L.fp8gemm_fill_uniform.restype = None
+    L.fp8gemm_fill_uniform.argtypes = [vp, ctypes.c_size_t, ci, ctypes.c_uint64, ctypes.c_float, ctypes.c_float]
+    L.fp8gemm_fill_normal.restype = None
+    L.fp8gemm_fill_normal.argtypes = [vp, ctypes.c_size_t, ci, ctypes.c_uint64, ctypes.c_float, ctypes.c_float]
+    L.fp8gemm_fill_weights.restype = None
+    L.fp8gemm_fill_weights.argtypes = [vp, ctypes.c_size_t, ci, ctypes.c_uint64, ctypes.c_float]
+    L.fp8gemm_fill_loguniform.restype = None
+    L.fp8gemm_fill_loguniform.argtypes = [vp, ctypes.c_size_t, ci, ctypes.c_uint64]
+    _lib = L
+    return L
+
+
+def check(code):
+    if code != 0:
+        raise Fp8GemmError("fp8gemm error %d: %s" % (code, lib().fp8gemm_error_string(code).decode()))
+
+
+# ---------------------------------------------------------------- host codec
+def encode(values, fmt):
+    """float32 numpy array -> uint8 codes (RNE, saturate to finite)."""
+    import numpy as np
+    values = np.ascontiguousarray(values, dtype=np.float32)
+    out = np.empty(values.shape, dtype=np.uint8)
+    lib().fp8gemm_encode(values.ctypes.data, out.ctypes.data, values.size, fmt)
+    return out
+
+
+def decode(codes, fmt):
+    import numpy as np
+    codes = np.ascontiguousarray(codes, dtype=np.uint8)
+    out = np.empty(codes.shape, dtype=np.float32)
+    lib().fp8gemm_decode(codes.ctypes.data, out.ctypes.data, codes.size, fmt)
+    return out
+
+
+def fill(shape, fmt, seed, dist="normal", **kw):
+    """Seeded synthetic fp8 matrix as a uint8 numpy array (host memory)."""
+    import numpy as np
+    out = np.empty(shape, dtype=np.uint8)
+    L = lib()
+    if dist == "normal":
+        L.fp8gemm_fill_normal(out.ctypes.data, out.size, fmt, seed, kw.get("mean", 0.0), kw.get("sigma", 1.0))
+    elif dist == "uniform":
+        L.fp8gemm_fill_uniform(out.ctypes.data, out.size, fmt, seed, kw.get("lo", -1.0), kw.get("hi", 1.0))
+    elif dist == "weights":
+        L.fp8gemm_fill_weights(out.ctypes.data, out.size, fmt, seed, kw.get("sigma", 0.02))
+    elif dist == "loguniform":
+        L.fp8gemm_fill_loguniform(out.ctypes.data, out.size, fmt, seed)
+    else:
+        raise ValueError(dist)
+    return out
+
+
+# ---------------------------------------------------------------- device GEMM
+def _fmt_of(t, fmt):
+    import torch
+    if fmt is not None:
+        return fmt
+    if t.dtype == torch.float8_e4m3fn:
+        return E4M3
+    if t.dtype == torch.float8_e5m2:
+        return E5M2
+    raise TypeError("operand must be float8_e4m3fn / float8_e5m2, or uint8 with an explicit format")
+
+
+def _stream_handle(stream):
+    import torch
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return ctypes.c_void_p(stream.cuda_stream)
+
+
+def gemm(a, b, out=None, a_fmt=None, b_fmt=None, stages=2, algo=ALGO_AUTO, variant=None,
+         split_k=0, stream=None):
+    """out[m, n] = sum_k a[m, k] * b[n, k] on the device holding a and b.
+
+    a: (m, k), b: (n, k) contiguous device tensors of fp8 (or uint8 + format);
+    out: (m, n) float32 device tensor, allocated when None.  Launches on
+    `stream` (default: torch's current stream) and does not synchronise.
+    """
+    import torch
+    if not (a.is_cuda and b.is_cuda):
+        raise Fp8GemmError("operands must live in device memory")
+    if not (a.is_contiguous() and b.is_contiguous()):
+        raise Fp8GemmError("operands must be contiguous")
+    m, k = a.shape
+    n, k2 = b.shape
+    if k != k2:
+        raise Fp8GemmError("inner dimensions differ: %d vs %d" % (k, k2))
+    fa, fb = _fmt_of(a, a_fmt), _fmt_of(b, b_fmt)
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    L = lib()
+    s = _stream_handle(stream)
+    if variant is None and split_k == 0:
+        code = L.fp8gemm_launch_algo(m, k, n, a.data_ptr(), fa, b.data_ptr(), fb, out.data_ptr(), stages, algo, s)
+    else:
+        code = L.fp8gemm_launch_tuned(m, k, n, a.data_ptr(), fa, b.data_ptr(), fb, out.data_ptr(), algo,
+                                      -1 if variant is None else variant, split_k, s)
+    check(code)
+    return out
+
+
+_PAIR = {(E4M3, E4M3): "e4m3_e4m3", (E5M2, E5M2): "e5m2_e5m2", (E4M3, E5M2): "e4m3_e5m2", (E5M2, E4M3): "e5m2_e4m3"}
+
+
+def _entry(m, k, n, a, b, out, stage):
+    fn = getattr(lib(), "fp8gemm_%s_stage%d" % (_PAIR[(_fmt_of(a, None), _fmt_of(b, None))], stage))
+    return fn(m, k, n, a.data_ptr(), b.data_ptr(), out.data_ptr())
+
+
+def GEMM(m, k, n, a, b, out):
+    """gemm::GEMM of the reference (gemm.cuh:12-15, 24-27, 36-39, 47-50): default
+    stream, returns the launch status."""
+    return _entry(m, k, n, a, b, out, 2)
+
+
+def GEMM4(m, k, n, a, b, out):
+    """gemm::GEMM4 of the reference (gemm.cuh:18-21, 30-33, 41-44, 52-55)."""
+    return _entry(m, k, n, a, b, out, 4)

@@ -1,0 +1,47 @@
+// Shared device-side vocabulary for the gfx950 FP8 GEMM kernels.
+#ifndef FP8GEMM_DEVICE_COMMON_H
+#define FP8GEMM_DEVICE_COMMON_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+#define FP8GEMM_WAVE 64
+
+// v_mfma_f32_32x32x64_f8f6f4: D(32x32 fp32) += A(32x64 fp8) * B(64x32 fp8).
+// AF / BF: 0 = E4M3, 1 = E5M2 (the instruction's cbsz / blgp fields).  Both
+// block-scale operands are literal zero, which selects the unscaled opcode.
+//
+// Operand layout: lane l supplies 32 bytes of row (l % 32) of A, respectively
+// of column (l % 32) of B, covering one K half chosen by (l / 32).  A and B use
+// the same lane->K map, so any K bytes may be given to a lane as long as the
+// A lane and the B lane of equal (l / 32) are given the same ones.
+// Result layout: register r of lane l holds D[8*(r/4) + 4*(l/32) + r%4][l%32].
+template <int AF, int BF>
+__device__ __forceinline__ v16f mfma_32x32x64(v8i a, v8i b, v16f c)
+{
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, AF, BF, 0, 0, 0, 0);
+}
+
+// v_mfma_f32_16x16x128_f8f6f4: D(16x16) += A(16x128) * B(128x16).  Lane l
+// supplies 32 bytes of row / column (l % 16), K quarter (l / 16); register r of
+// lane l holds D[4*(l/16) + r][l%16].
+template <int AF, int BF>
+__device__ __forceinline__ v4f mfma_16x16x128(v8i a, v8i b, v4f c)
+{
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, AF, BF, 0, 0, 0, 0);
+}
+
+__device__ __forceinline__ v8i pack8(v4i lo, v4i hi)
+{
+    v8i r;
+    r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+    r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+    return r;
+}
+
+#endif  // FP8GEMM_DEVICE_COMMON_H

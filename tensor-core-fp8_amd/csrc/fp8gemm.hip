@@ -1,0 +1,366 @@
+// C ABI, argument validation and kernel selection of the gfx950 FP8 GEMM
+// library.  The entry points are declared in include/fp8gemm.h; together they
+// stand where the launch functions of the reference stand
+// (GEMM/include/gemm.cuh:11-55, defined at GEMM/src/gemm.cu:263-285 and
+// siblings): validate, pick a kernel, launch asynchronously, return the launch
+// status.
+#include "fp8gemm.h"
+
+#include <hip/hip_runtime.h>
+
+#include <mutex>
+
+#include "kernel_direct.h"
+#include "kernel_skinny.h"
+#include "kernel_tile.h"
+
+namespace {
+
+constexpr int kVersion = 100;
+constexpr int kMaxDevices = 64;
+
+// ------------------------------------------------------------------ variants
+// Tiled kernel shapes: <BM, BN, BK, waves_m, waves_n, stages, swizzle>.
+using TileA = TileShape<256, 256, 128, 2, 2, 2, 3>;   // 4 waves, 128x128 per wave, 128 KiB LDS
+using TileB = TileShape<256, 256, 64, 2, 2, 4, 3>;    // same tile, 4 x 32 KiB stages
+using TileC = TileShape<256, 256, 128, 2, 4, 2, 3>;   // 8 waves, 128x64 per wave
+using TileD = TileShape<256, 256, 64, 2, 4, 4, 3>;
+using TileE = TileShape<128, 128, 128, 2, 2, 2, 3>;   // small tile for small problems
+using TileF = TileShape<128, 128, 128, 2, 2, 4, 3>;
+constexpr int kNumTileVariants = 6;
+
+// Skinny kernel shapes: <MT, TN, BK, stages>.
+template <int MT, int TN>
+using SkinnyV0 = SkinnyShape<MT, TN, 128, 5>;
+template <int MT, int TN>
+using SkinnyV1 = SkinnyShape<MT, TN, 256, 4>;
+template <int MT, int TN>
+using SkinnyV2 = SkinnyShape<MT, TN, 128, 8>;
+template <int MT, int TN>
+using SkinnyV3 = SkinnyShape<MT, TN, 256, 6>;
+constexpr int kNumSkinnyVariants = 4;
+
+struct Scratch {
+    void *ptr = nullptr;
+    size_t bytes = 0;
+};
+Scratch g_scratch[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+hipError_t scratch_get(size_t bytes, void **out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    Scratch &s = g_scratch[dev];
+    if (s.bytes < bytes) {
+        if (s.ptr) {
+            // earlier launches may still be reading the old buffer
+            e = hipDeviceSynchronize();
+            if (e != hipSuccess) return e;
+            (void)hipFree(s.ptr);
+            s.ptr = nullptr;
+            s.bytes = 0;
+        }
+        e = hipMalloc(&s.ptr, bytes);
+        if (e != hipSuccess) {
+            s.ptr = nullptr;
+            return e;
+        }
+        s.bytes = bytes;
+    }
+    *out = s.ptr;
+    return hipSuccess;
+}
+
+template <class Kernel>
+hipError_t allow_lds(Kernel kernel, int bytes)
+{
+    if (bytes <= 64 * 1024) return hipSuccess;
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
+// ------------------------------------------------------------------ direct
+template <int AF, int BF>
+hipError_t launch_direct(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
+                         hipStream_t stream)
+{
+    const long gy = (m + 31) / 32, gx = (n + 31) / 32;
+    if (gy > 65535) return hipErrorInvalidValue;
+    const bool vec_ok = (k % 16 == 0) && ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) % 16 == 0);
+    hipLaunchKernelGGL((gemm_direct_kernel<AF, BF>), dim3((unsigned)gx, (unsigned)gy), dim3(64), 0, stream,
+                       m, k, n, a, b, out, vec_ok ? 1 : 0);
+    return hipGetLastError();
+}
+
+// ------------------------------------------------------------------ tiled
+template <class S, int AF, int BF>
+hipError_t launch_tile_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
+                             hipStream_t stream)
+{
+    if (k % S::BK != 0) return hipErrorInvalidValue;
+    const int tiles_m = (m + S::BM - 1) / S::BM;
+    const int tiles_n = (n + S::BN - 1) / S::BN;
+    // XCD-local super-blocks of tiles: 32 CUs per XCD -> blocks of up to 32 tiles,
+    // shaped to balance A-panel and B-panel reuse.
+    int GM = 4, GN = 8;
+    if (tiles_m < GM) { GM = tiles_m; }
+    if (tiles_n < GN) { GN = tiles_n; }
+    const int nb = ((tiles_m + GM - 1) / GM) * ((tiles_n + GN - 1) / GN);
+    const long grid = (long)((nb + 7) / 8) * 8 * GM * GN;
+    auto kernel = gemm_tile_kernel<S, AF, BF>;
+    hipError_t e = allow_lds(kernel, S::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(S::THREADS), S::LDS_BYTES, stream,
+                       m, k, n, a, b, out, tiles_m, tiles_n, GM, GN);
+    return hipGetLastError();
+}
+
+template <int AF, int BF>
+hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
+                       int variant, hipStream_t stream)
+{
+    switch (variant) {
+    case 0: return launch_tile_shape<TileA, AF, BF>(m, k, n, a, b, out, stream);
+    case 1: return launch_tile_shape<TileB, AF, BF>(m, k, n, a, b, out, stream);
+    case 2: return launch_tile_shape<TileC, AF, BF>(m, k, n, a, b, out, stream);
+    case 3: return launch_tile_shape<TileD, AF, BF>(m, k, n, a, b, out, stream);
+    case 4: return launch_tile_shape<TileE, AF, BF>(m, k, n, a, b, out, stream);
+    case 5: return launch_tile_shape<TileF, AF, BF>(m, k, n, a, b, out, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+// ------------------------------------------------------------------ skinny
+struct SkinnyPlan {
+    int mt, tn, variant, nsplit;
+};
+
+template <class S, int AF, int BF>
+hipError_t launch_skinny_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
+                               int nsplit, hipStream_t stream)
+{
+    if (m > S::MP || n % S::NP != 0 || nsplit < 1 || k % nsplit != 0 || (k / nsplit) % S::BK != 0)
+        return hipErrorInvalidValue;
+    const int ngroups = n / S::NP;
+    const int kchunk = k / nsplit;
+    float *dst = out;
+    if (nsplit > 1) {
+        void *ws = nullptr;
+        hipError_t e = scratch_get((size_t)nsplit * m * n * sizeof(float), &ws);
+        if (e != hipSuccess) return e;
+        dst = static_cast<float *>(ws);
+    }
+    auto kernel = gemm_skinny_kernel<S, AF, BF>;
+    hipError_t e = allow_lds(kernel, S::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(ngroups * nsplit)), dim3(64), S::LDS_BYTES, stream,
+                       m, k, n, a, b, dst, ngroups, kchunk);
+    e = hipGetLastError();
+    if (e != hipSuccess || nsplit == 1) return e;
+    const size_t count = (size_t)m * n;
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
+                       dst, out, count, nsplit);
+    return hipGetLastError();
+}
+
+template <template <int, int> class V, int AF, int BF>
+hipError_t launch_skinny_mt(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
+                            const SkinnyPlan &p, hipStream_t stream)
+{
+#define SK(MT, TN) \
+    if (p.mt == MT && p.tn == TN) return launch_skinny_shape<V<MT, TN>, AF, BF>(m, k, n, a, b, out, p.nsplit, stream);
+    SK(1, 1) SK(1, 2) SK(1, 4)
+    SK(2, 1) SK(2, 2) SK(2, 4)
+    SK(3, 1) SK(3, 2) SK(3, 4)
+    SK(4, 1) SK(4, 2) SK(4, 4)
+#undef SK
+    return hipErrorInvalidValue;
+}
+
+template <int AF, int BF>
+hipError_t launch_skinny(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
+                         const SkinnyPlan &p, hipStream_t stream)
+{
+    switch (p.variant) {
+    case 0: return launch_skinny_mt<SkinnyV0, AF, BF>(m, k, n, a, b, out, p, stream);
+    case 1: return launch_skinny_mt<SkinnyV1, AF, BF>(m, k, n, a, b, out, p, stream);
+    case 2: return launch_skinny_mt<SkinnyV2, AF, BF>(m, k, n, a, b, out, p, stream);
+    case 3: return launch_skinny_mt<SkinnyV3, AF, BF>(m, k, n, a, b, out, p, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+bool skinny_ok(int m, int k, int n)
+{
+    return m <= 64 && n % 16 == 0 && k % 256 == 0;
+}
+
+// Picks columns per wave, LDS shape and split-K factor so that the number of
+// independent streams is close to a multiple of the CU count and every stream
+// is long enough to amortise its start-up.
+SkinnyPlan plan_skinny(int m, int k, int n)
+{
+    SkinnyPlan p;
+    p.mt = (m + 15) / 16;
+    p.variant = 1;
+    int tn = (p.mt >= 3) ? 4 : p.mt;              // keep A traffic <= B traffic
+    while (tn > 1 && n % (16 * tn) != 0) tn /= 2;
+    p.tn = tn;
+    const int groups = n / (16 * tn);
+    const int ksteps = k / 256;
+    constexpr int kCUs = 256;
+    int best = 1;
+    double best_score = -1.0;
+    for (int s = 1; s <= 16; ++s) {
+        if (ksteps % s != 0 || ksteps / s < 4) continue;
+        const long units = (long)groups * s;
+        const long rounds = (units + kCUs - 1) / kCUs;
+        double eff = (double)units / (double)(rounds * kCUs);   // tail balance
+        if (rounds < 2) eff *= 0.5 + 0.25 * rounds;             // too few streams per CU
+        if (rounds > 8) eff *= 0.9;                             // more than LDS can hold at once
+        const double score = eff - 0.03 * (s - 1);              // reduction pass is not free
+        if (score > best_score) { best_score = score; best = s; }
+    }
+    p.nsplit = best;
+    return p;
+}
+
+int select_algo(int m, int k, int n)
+{
+    if (skinny_ok(m, k, n)) return FP8GEMM_ALGO_SKINNY;
+    if (k % 128 == 0) return FP8GEMM_ALGO_TILE;
+    return FP8GEMM_ALGO_DIRECT;
+}
+
+int default_tile_variant(int m, int n, int stages)
+{
+    const long tiles256 = (long)((m + 255) / 256) * ((n + 255) / 256);
+    if (tiles256 < 256) return stages == 2 ? 4 : 5;   // small problem: 128x128 tiles fill more CUs
+    return stages == 2 ? 0 : 1;
+}
+
+template <int AF, int BF>
+hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out, int stages,
+                    int algo, int variant, int nsplit, hipStream_t stream)
+{
+    const bool aligned = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) % 16) == 0;
+    if (algo == FP8GEMM_ALGO_AUTO) {
+        algo = select_algo(m, k, n);
+        if (!aligned) algo = FP8GEMM_ALGO_DIRECT;
+    }
+    switch (algo) {
+    case FP8GEMM_ALGO_DIRECT:
+        return launch_direct<AF, BF>(m, k, n, a, b, out, stream);
+    case FP8GEMM_ALGO_TILE:
+        if (!aligned || k % 128 != 0) return hipErrorInvalidValue;
+        if (variant < 0) variant = default_tile_variant(m, n, stages);
+        return launch_tile<AF, BF>(m, k, n, a, b, out, variant, stream);
+    case FP8GEMM_ALGO_SKINNY: {
+        if (!aligned || !skinny_ok(m, k, n)) return hipErrorInvalidValue;
+        SkinnyPlan p = plan_skinny(m, k, n);
+        if (variant >= 0) {
+            // tuning hook: variant = shape_index + 16 * columns-per-wave/16 (0 keeps the plan's)
+            p.variant = variant % 16;
+            if (variant / 16 > 0) p.tn = variant / 16;
+        }
+        if (nsplit > 0) p.nsplit = nsplit;
+        return launch_skinny<AF, BF>(m, k, n, a, b, out, p, stream);
+    }
+    default:
+        return hipErrorInvalidValue;
+    }
+}
+
+int launch_checked(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt, float *out,
+                   int stages, int algo, int variant, int nsplit, void *stream)
+{
+    if (m <= 0 || k <= 0 || n <= 0 || !a || !b || !out) return (int)hipErrorInvalidValue;
+    if ((a_fmt != FP8GEMM_E4M3 && a_fmt != FP8GEMM_E5M2) || (b_fmt != FP8GEMM_E4M3 && b_fmt != FP8GEMM_E5M2))
+        return (int)hipErrorInvalidValue;
+    if (stages != 2 && stages != 4) return (int)hipErrorInvalidValue;
+    if (algo < FP8GEMM_ALGO_AUTO || algo > FP8GEMM_ALGO_SKINNY) return (int)hipErrorInvalidValue;
+    const uint8_t *pa = static_cast<const uint8_t *>(a);
+    const uint8_t *pb = static_cast<const uint8_t *>(b);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e;
+    if (a_fmt == FP8GEMM_E4M3 && b_fmt == FP8GEMM_E4M3)
+        e = dispatch<0, 0>(m, k, n, pa, pb, out, stages, algo, variant, nsplit, s);
+    else if (a_fmt == FP8GEMM_E5M2 && b_fmt == FP8GEMM_E5M2)
+        e = dispatch<1, 1>(m, k, n, pa, pb, out, stages, algo, variant, nsplit, s);
+    else if (a_fmt == FP8GEMM_E4M3)
+        e = dispatch<0, 1>(m, k, n, pa, pb, out, stages, algo, variant, nsplit, s);
+    else
+        e = dispatch<1, 0>(m, k, n, pa, pb, out, stages, algo, variant, nsplit, s);
+    return (int)e;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fp8gemm_launch(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
+                   float *out, int stages, void *stream)
+{
+    return launch_checked(m, k, n, a, a_fmt, b, b_fmt, out, stages, FP8GEMM_ALGO_AUTO, -1, 0, stream);
+}
+
+int fp8gemm_launch_algo(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
+                        float *out, int stages, int algo, void *stream)
+{
+    return launch_checked(m, k, n, a, a_fmt, b, b_fmt, out, stages, algo, -1, 0, stream);
+}
+
+int fp8gemm_launch_tuned(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
+                         float *out, int algo, int variant, int split_k, void *stream)
+{
+    return launch_checked(m, k, n, a, a_fmt, b, b_fmt, out, 2, algo, variant, split_k, stream);
+}
+
+int fp8gemm_num_variants(int algo)
+{
+    if (algo == FP8GEMM_ALGO_TILE) return kNumTileVariants;
+    if (algo == FP8GEMM_ALGO_SKINNY) return kNumSkinnyVariants;
+    return algo == FP8GEMM_ALGO_DIRECT ? 1 : 0;
+}
+
+int fp8gemm_select_algo(int m, int k, int n)
+{
+    if (m <= 0 || k <= 0 || n <= 0) return -1;
+    return select_algo(m, k, n);
+}
+
+size_t fp8gemm_scratch_bytes(int m, int k, int n)
+{
+    if (m <= 0 || k <= 0 || n <= 0 || select_algo(m, k, n) != FP8GEMM_ALGO_SKINNY) return 0;
+    const SkinnyPlan p = plan_skinny(m, k, n);
+    return p.nsplit > 1 ? (size_t)p.nsplit * m * n * sizeof(float) : 0;
+}
+
+const char *fp8gemm_error_string(int code)
+{
+    return hipGetErrorString(static_cast<hipError_t>(code));
+}
+
+int fp8gemm_version(void) { return kVersion; }
+
+#define FP8GEMM_ENTRY(NAME, AFMT, BFMT, STAGES)                                              \
+    int NAME(int m, int k, int n, const void *a, const void *b, float *out)                  \
+    {                                                                                        \
+        return launch_checked(m, k, n, a, AFMT, b, BFMT, out, STAGES, FP8GEMM_ALGO_AUTO, -1, \
+                              0, nullptr);                                                   \
+    }
+
+FP8GEMM_ENTRY(fp8gemm_e4m3_e4m3_stage2, FP8GEMM_E4M3, FP8GEMM_E4M3, 2)
+FP8GEMM_ENTRY(fp8gemm_e4m3_e4m3_stage4, FP8GEMM_E4M3, FP8GEMM_E4M3, 4)
+FP8GEMM_ENTRY(fp8gemm_e5m2_e5m2_stage2, FP8GEMM_E5M2, FP8GEMM_E5M2, 2)
+FP8GEMM_ENTRY(fp8gemm_e5m2_e5m2_stage4, FP8GEMM_E5M2, FP8GEMM_E5M2, 4)
+FP8GEMM_ENTRY(fp8gemm_e4m3_e5m2_stage2, FP8GEMM_E4M3, FP8GEMM_E5M2, 2)
+FP8GEMM_ENTRY(fp8gemm_e4m3_e5m2_stage4, FP8GEMM_E4M3, FP8GEMM_E5M2, 4)
+FP8GEMM_ENTRY(fp8gemm_e5m2_e4m3_stage2, FP8GEMM_E5M2, FP8GEMM_E4M3, 2)
+FP8GEMM_ENTRY(fp8gemm_e5m2_e4m3_stage4, FP8GEMM_E5M2, FP8GEMM_E4M3, 4)
+
+}  // extern "C"

@@ -1,0 +1,153 @@
+"""GPU parity: the HIP kernels, called through the C ABI, against the CPU oracle.
+
+Bar (the reference's own CPU fp32 loop, GEMM/gemm_main.cpp:39-53, is the truth):
+  |C_gpu - C_ref| <= 2*K*2^-24 * sum_k |a_ik * b_kj|   per element,
+and bit-exact wherever no rounding can occur.
+"""
+import zlib
+
+import numpy as np
+import pytest
+
+from conftest import finite_codes, random_codes
+
+pytestmark = pytest.mark.gpu
+
+PAIRS = [(0, 0), (1, 1), (0, 1), (1, 0)]
+ALGOS = {"direct": 1, "tile": 2, "skinny": 3}
+
+
+def run_gpu(pkg, A, fa, B, fb, **kw):
+    import torch
+    dA = torch.from_numpy(A).cuda()
+    dB = torch.from_numpy(B).cuda()
+    out = torch.full((A.shape[0], B.shape[0]), float("nan"), dtype=torch.float32, device="cuda")
+    pkg.gemm(dA, dB, out=out, a_fmt=fa, b_fmt=fb, **kw)
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def mfma_window_term(oracle, A, fa, B, fb, block=64):
+    """Extra error the f8f6f4 MFMA can add on top of reordered fp32 summation.
+
+    Measured on MI355X: inside one MFMA the products of a K block are aligned to
+    the largest product exponent of the block and only ~14 bits below it are
+    kept (2^16 + 2^3 survives, 2^16 + 2^2 does not); between MFMAs the sum is
+    plain fp32.  So each block can lose up to one unit of 2^-13 * max|product|
+    per product.
+    """
+    a = oracle.decode(A, fa).astype(np.float64)
+    b = oracle.decode(B, fb).astype(np.float64)
+    M, K = a.shape
+    N = b.shape[0]
+    term = np.zeros((M, N))
+    for k0 in range(0, K, block):
+        pa = np.abs(a[:, None, k0:k0 + block])
+        pb = np.abs(b[None, :, k0:k0 + block])
+        term += (pa * pb).max(axis=2) * min(block, K - k0)
+    return term * 2.0 ** -13
+
+
+def assert_within_bound(oracle, C, A, fa, B, fb, rows=None, hw_term=False):
+    K = A.shape[1]
+    Cref, S = oracle.gemm(A, fa, B, fb, rows=rows, with_scale=True)
+    got = C if rows is None else C[rows]
+    assert np.isfinite(got).all()
+    err = np.abs(got.astype(np.float64) - Cref.astype(np.float64))
+    tol = oracle.tolerance(K, S)
+    if hw_term:
+        tol = tol + mfma_window_term(oracle, A, fa, B, fb)
+    worst = float((err / np.maximum(tol, 1e-300)).max())
+    assert (err <= tol).all(), "worst err/tol = %g" % worst
+    return worst
+
+
+SHAPES = [
+    ("direct", (128, 128, 128)), ("direct", (37, 100, 53)), ("direct", (1, 1, 1)), ("direct", (65, 17, 33)),
+    ("direct", (40, 1030, 70)),
+    ("tile", (128, 128, 128)), ("tile", (256, 384, 512)), ("tile", (300, 256, 200)), ("tile", (512, 1024, 768)),
+    ("tile", (1, 128, 1)),
+    ("skinny", (16, 256, 64)), ("skinny", (1, 512, 128)), ("skinny", (13, 1024, 256)), ("skinny", (64, 512, 192)),
+    ("skinny", (33, 2048, 80)),
+]
+
+
+@pytest.mark.parametrize("fa,fb", PAIRS)
+@pytest.mark.parametrize("algo,shape", SHAPES)
+def test_all_finite_codes(pkg, oracle, fa, fb, algo, shape):
+    """Operands drawn uniformly from every finite code (subnormals, extremes, -0): the
+    widest dynamic range the formats allow.  Bound = the fp32 reordering bound plus
+    the MFMA alignment-window term measured for the hardware."""
+    M, K, N = shape
+    rng = np.random.default_rng(zlib.crc32(repr((fa, fb, algo, shape)).encode()))
+    A = random_codes(rng, (M, K), fa)
+    B = random_codes(rng, (N, K), fb)
+    # keep e5m2 magnitudes below 2^10 so that fp32 sums cannot overflow
+    if fa == 1:
+        A = np.where(((A >> 2) & 0x1F) > 24, A & 0x83 | 0x3C, A).astype(np.uint8)
+    if fb == 1:
+        B = np.where(((B >> 2) & 0x1F) > 24, B & 0x83 | 0x3C, B).astype(np.uint8)
+    C = run_gpu(pkg, A, fa, B, fb, algo=ALGOS[algo])
+    assert_within_bound(oracle, C, A, fa, B, fb, hw_term=True)
+
+
+@pytest.mark.parametrize("fa,fb", PAIRS)
+@pytest.mark.parametrize("algo,shape", [
+    ("direct", (64, 2048, 96)), ("tile", (256, 2048, 256)), ("tile", (384, 4096, 640)),
+    ("skinny", (16, 4096, 512)), ("skinny", (64, 2048, 256)), ("skinny", (1, 8192, 256)),
+])
+def test_normal_inputs_within_fp32_reordering_bound(pkg, oracle, fa, fb, algo, shape):
+    """4*N(0,1) inputs (the four-pairings workload) against the plain bound
+    |C_gpu - C_ref| <= 2*K*2^-24 * sum_k |a*b|."""
+    M, K, N = shape
+    A = pkg.fill((M, K), fa, seed=0xA11CE + K, dist="normal", sigma=4.0)
+    B = pkg.fill((N, K), fb, seed=0xB0B + K, dist="normal", sigma=4.0)
+    C = run_gpu(pkg, A, fa, B, fb, algo=ALGOS[algo])
+    worst = assert_within_bound(oracle, C, A, fa, B, fb)
+    assert worst < 0.25
+
+
+@pytest.mark.parametrize("fa,fb", PAIRS)
+@pytest.mark.parametrize("algo", ["direct", "tile", "skinny"])
+def test_decode_through_mfma_is_bit_exact(pkg, oracle, fa, fb, algo):
+    """One-hot A with value 1.0 selects single entries of B: C[i, j] == decode(B[j, k_i])
+    exactly, for every finite code, and likewise with the roles swapped."""
+    one = {0: 0x38, 1: 0x3C}
+    K = 256
+    M = 64 if algo == "skinny" else 256
+    N = 256
+    rng = np.random.default_rng(7)
+    ks = rng.permutation(K)[:M] if M <= K else rng.integers(0, K, M)
+    A = np.zeros((M, K), dtype=np.uint8)
+    A[np.arange(M), ks] = one[fa]
+    codes = finite_codes(fb)
+    B = codes[rng.integers(0, codes.size, (N, K))]
+    B[:, ks[0]] = np.resize(codes, N)            # every finite code appears at least once
+    C = run_gpu(pkg, A, fa, B, fb, algo=ALGOS[algo])
+    expect = oracle.decode(B, fb)[:, ks].T       # (M, N)
+    assert np.array_equal(C.view(np.uint32) & 0x7FFFFFFF, expect.view(np.uint32) & 0x7FFFFFFF)
+    assert np.array_equal(C, expect)
+    # swapped roles: one-hot B selects entries of A
+    if algo != "skinny":
+        A2 = finite_codes(fa)[rng.integers(0, finite_codes(fa).size, (M, K))]
+        B2 = np.zeros((N, K), dtype=np.uint8)
+        kn = rng.integers(0, K, N)
+        B2[np.arange(N), kn] = one[fb]
+        C2 = run_gpu(pkg, A2, fa, B2, fb, algo=ALGOS[algo])
+        assert np.array_equal(C2, oracle.decode(A2, fa)[:, kn])
+
+
+@pytest.mark.parametrize("algo,shape", [("direct", (96, 200, 64)), ("tile", (256, 1024, 256)), ("skinny", (48, 1024, 128))])
+def test_small_integers_are_exact(pkg, oracle, algo, shape):
+    """|values| <= 8 and K <= 2^10: every partial sum is an integer below 2^24, so any
+    summation order gives the same bits as the oracle."""
+    M, K, N = shape
+    rng = np.random.default_rng(11)
+    vals = np.arange(-8, 9, dtype=np.float32)
+    A = oracle.encode(vals[rng.integers(0, vals.size, (M, K))], 0)
+    B = oracle.encode(vals[rng.integers(0, vals.size, (N, K))], 1)
+    C = run_gpu(pkg, A, 0, B, 1, algo=ALGOS[algo])
+    Cref = oracle.gemm(A, 0, B, 1)
+    assert np.array_equal(C, Cref)
+    ints = oracle.decode(A, 0).astype(np.int64) @ oracle.decode(B, 1).astype(np.int64).T
+    assert np.array_equal(C.astype(np.int64), ints)
