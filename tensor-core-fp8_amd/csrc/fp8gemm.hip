@@ -11,6 +11,7 @@
 #include <mutex>
 
 #include "kernel_direct.h"
+#include "kernel_ptile.h"
 #include "kernel_skinny.h"
 #include "kernel_tile.h"
 
@@ -18,16 +19,16 @@ namespace {
 
 constexpr int kVersion = 100;
 constexpr int kMaxDevices = 64;
+constexpr int kDefaultStagger = 1;    // units of ~2048 clocks between phase groups of the persistent kernel
 
 // ------------------------------------------------------------------ variants
 // Tiled kernel shapes: <BM, BN, BK, waves_m, waves_n, stages, swizzle>.
-using TileA = TileShape<256, 256, 128, 2, 2, 2, 3>;   // 4 waves, 128x128 per wave, 128 KiB LDS
-using TileB = TileShape<256, 256, 64, 2, 2, 4, 3>;    // same tile, 4 x 32 KiB stages
-using TileC = TileShape<256, 256, 128, 2, 4, 2, 3>;   // 8 waves, 128x64 per wave
-using TileD = TileShape<256, 256, 64, 2, 4, 4, 3>;
-using TileE = TileShape<128, 128, 128, 2, 2, 2, 3>;   // small tile for small problems
-using TileF = TileShape<128, 128, 128, 2, 2, 4, 3>;
-constexpr int kNumTileVariants = 6;
+using TileP2 = TileShape<256, 256, 128, 2, 2, 2, 3>;  // persistent, 2 x 64 KiB ring, 128x128 per wave
+using TileP4 = TileShape<256, 256, 64, 2, 2, 4, 2>;   // persistent, 4 x 32 KiB ring
+using TileP8 = TileShape<256, 256, 128, 2, 4, 2, 3>;  // persistent, 8 waves, 128x64 per wave
+using TileS2 = TileShape<128, 128, 128, 2, 2, 2, 3>;  // one tile per workgroup, for small problems
+using TileS4 = TileShape<128, 128, 128, 2, 2, 4, 3>;
+constexpr int kNumTileVariants = 5;               // 0 P2, 1 P4, 2 P8, 3 S2, 4 S4
 
 // Skinny kernel shapes: <MT, TN, BK, stages>.
 template <int MT, int TN>
@@ -119,17 +120,40 @@ hipError_t launch_tile_shape(int m, int k, int n, const uint8_t *a, const uint8_
     return hipGetLastError();
 }
 
+// persistent form: one workgroup per CU walks the tiles of its XCD
+template <class S, int AF, int BF>
+hipError_t launch_ptile_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
+                              hipStream_t stream)
+{
+    if (k % S::BK != 0) return hipErrorInvalidValue;
+    const int tiles_m = (m + S::BM - 1) / S::BM;
+    const int tiles_n = (n + S::BN - 1) / S::BN;
+    int GM = 4, GN = 8;                       // 32 tiles = the 32 CUs of one XCD
+    if (tiles_m < GM) { GM = tiles_m; }
+    if (tiles_n < GN) { GN = tiles_n; }
+    const int nb = ((tiles_m + GM - 1) / GM) * ((tiles_n + GN - 1) / GN);
+    const int rounds = (nb + 7) / 8;
+    const int grid = 8 * GM * GN;
+    // phase stagger only pays when a workgroup has several tiles to write
+    const int stagger = rounds >= 2 ? kDefaultStagger : 0;
+    auto kernel = gemm_ptile_kernel<S, AF, BF>;
+    hipError_t e = allow_lds(kernel, S::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(S::THREADS), S::LDS_BYTES, stream,
+                       m, k, n, a, b, out, tiles_m, tiles_n, GM, GN, rounds, stagger);
+    return hipGetLastError();
+}
+
 template <int AF, int BF>
 hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
                        int variant, hipStream_t stream)
 {
     switch (variant) {
-    case 0: return launch_tile_shape<TileA, AF, BF>(m, k, n, a, b, out, stream);
-    case 1: return launch_tile_shape<TileB, AF, BF>(m, k, n, a, b, out, stream);
-    case 2: return launch_tile_shape<TileC, AF, BF>(m, k, n, a, b, out, stream);
-    case 3: return launch_tile_shape<TileD, AF, BF>(m, k, n, a, b, out, stream);
-    case 4: return launch_tile_shape<TileE, AF, BF>(m, k, n, a, b, out, stream);
-    case 5: return launch_tile_shape<TileF, AF, BF>(m, k, n, a, b, out, stream);
+    case 0: return launch_ptile_shape<TileP2, AF, BF>(m, k, n, a, b, out, stream);
+    case 1: return launch_ptile_shape<TileP4, AF, BF>(m, k, n, a, b, out, stream);
+    case 2: return launch_ptile_shape<TileP8, AF, BF>(m, k, n, a, b, out, stream);
+    case 3: return launch_tile_shape<TileS2, AF, BF>(m, k, n, a, b, out, stream);
+    case 4: return launch_tile_shape<TileS4, AF, BF>(m, k, n, a, b, out, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -239,7 +263,7 @@ int select_algo(int m, int k, int n)
 int default_tile_variant(int m, int n, int stages)
 {
     const long tiles256 = (long)((m + 255) / 256) * ((n + 255) / 256);
-    if (tiles256 < 256) return stages == 2 ? 4 : 5;   // small problem: 128x128 tiles fill more CUs
+    if (tiles256 < 192) return stages == 2 ? 3 : 4;   // small problem: 128x128 tiles fill more CUs
     return stages == 2 ? 0 : 1;
 }
 

@@ -1,0 +1,375 @@
+// Persistent LDS-tiled MFMA kernel for compute-bound shapes.
+//
+// The grid is one workgroup per CU; every workgroup walks a list of BM x BN
+// tiles of C.  Inside a tile the K loop is a software pipeline with three
+// levels, all of them explicit:
+//   * global -> LDS: 128-bit buffer loads that write LDS directly
+//     (buffer_load_dwordx4 ... lds) into a ring of STAGES buffers, issued
+//     STAGES-1 K tiles ahead of their use; no registers involved;
+//   * LDS -> registers: the operand fragments of K step u+1 are read while the
+//     MFMAs of K step u issue (two fragment sets, ping-pong);
+//   * registers -> C of tile i overlaps the first global loads of tile i+1.
+// One workgroup barrier per K tile, placed after the last fragment read of the
+// tile so that the MFMAs already issued keep the matrix pipe busy across it.
+//
+// The instruction order of a K step is fixed by hand: after every MFMA come at
+// most one global->LDS load and one or two fragment reads, so that the single
+// wave of a SIMD never makes the matrix pipe wait behind a block of memory
+// instructions and the texture-address unit sees an even stream (four waves x
+// one 1 KiB load per MFMA slot is its full rate of 64 B/clk).
+//
+// MFMA operand roles are swapped (src0 = B rows, src1 = A rows): the result
+// registers of a lane are then 4 consecutive columns of one row of C, which
+// turns the epilogue into 128-bit stores.
+//
+// LDS layout, swizzle and the K-permutation freedom are as in kernel_tile.h.
+// Requirements checked by the host: K % 128 == 0, 16-byte aligned a and b.
+#ifndef FP8GEMM_KERNEL_PTILE_H
+#define FP8GEMM_KERNEL_PTILE_H
+
+#include <type_traits>
+
+#include "kernel_tile.h"
+
+// s_waitcnt on the LDS/scalar counter only
+__device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xC07F); }
+
+// One wave-wide 16-byte-per-lane load from a buffer straight into LDS at
+// lds_addr + lane*16.  rsrc: buffer resource (SGPRs), voff: per-lane byte offset,
+// soff: uniform byte offset.  Bytes outside the buffer's extent read as zero.
+// Written as inline assembly so that the compiler does not order it against the
+// fragment reads (they never touch the ring slot being filled; the barrier
+// protocol guarantees it).  Completion is tracked with wait_vmcnt by hand.
+__device__ __forceinline__ void buffer_load_lds_b128(v4i rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+                 : "m0");
+}
+
+// 16-byte-per-lane store whose data operand stays in accumulation registers
+// (the MFMA results live there; a store can read them directly, a copy to
+// ordinary vector registers first would need 256 more registers per lane).
+__device__ __forceinline__ void global_store_b128_acc(void *uniform_base, uint32_t lane_off, v4f data)
+{
+    asm volatile("global_store_dwordx4 %0, %1, %2" : : "v"(lane_off), "a"(data), "s"(uniform_base) : "memory");
+}
+
+__device__ __forceinline__ v4i make_buffer_resource(const void *base, unsigned long long bytes)
+{
+    const unsigned long long a = reinterpret_cast<unsigned long long>(base);
+    const uint32_t extent = bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t)bytes;
+    v4i r;
+    r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
+    r[1] = __builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xFFFFu));   // stride 0
+    r[2] = __builtin_amdgcn_readfirstlane((int)extent);
+    r[3] = 0x00020000;                                                             // raw 32-bit data format
+    return r;
+}
+
+// DBG (tuning builds only, results are then wrong on purpose): bit 0 drops the
+// global loads, bit 1 the waits and barriers, bit 2 the fragment reads.
+template <class S, int AF, int BF, int DBG = 0>
+__global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, int N,
+                                                                 const uint8_t *__restrict__ A,
+                                                                 const uint8_t *__restrict__ B,
+                                                                 float *__restrict__ C,
+                                                                 int tiles_m, int tiles_n, int GM, int GN,
+                                                                 int rounds, int stagger)
+{
+    constexpr int BM = S::BM, BN = S::BN, BK = S::BK, CH = S::CH, RPI = S::RPI;
+    constexpr int STAGES = S::STAGES, TM = S::TM, TN = S::TN, KSTEPS = S::KSTEPS;
+    constexpr int NMFMA = TM * TN;
+    constexpr int NREADS = 2 * (TM + TN);          // ds_read_b128 per K step
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(LDS_AS uint8_t *)lds;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / S::WN;
+    const int wn = wave % S::WN;
+
+    // lane constants of the load plan and the fragment plan
+    const int lrow = lane / CH;
+    const int lslot = lane % CH;
+    const int fi = lane & 31;
+    const int fg = lane >> 5;
+    const int sw = tile_swizzle<BK, S::SWZ>(fi);
+    uint32_t frag_off[KSTEPS][2];
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) frag_off[s][j] = (uint32_t)(((s * 4 + 2 * fg + j) ^ sw) * 16);
+    const uint32_t a_base = (uint32_t)(wm * (BM / S::WM) + fi) * BK;
+    const uint32_t b_base = (uint32_t)(BM * BK) + (uint32_t)(wn * (BN / S::WN) + fi) * BK;
+    const int T = K / BK;
+
+    // workgroups with equal id mod 8 share an XCD (and its L2): XCD x takes the
+    // super-blocks x*rounds .. x*rounds+rounds-1, slot q of its 32 workgroups
+    // takes tile q of each super-block
+    const int xcd = blockIdx.x & 7;
+    const int slot = blockIdx.x >> 3;
+    const int nb_n = (tiles_n + GN - 1) / GN;
+    const int nb_total = ((tiles_m + GM - 1) / GM) * nb_n;
+
+    auto tile_of_round = [&](int r, int &tm, int &tn) -> bool {
+        const int blk = xcd * rounds + r;
+        if (r >= rounds || blk >= nb_total || slot >= GM * GN) return false;
+        tm = (blk / nb_n) * GM + slot / GN;
+        tn = (blk % nb_n) * GN + slot % GN;
+        return tm < tiles_m && tn < tiles_n;
+    };
+
+    // Global -> LDS load plan: one buffer resource per operand and tile (base =
+    // first row of the tile, extent = what is left of the matrix), a
+    // loop-invariant 32-bit offset per load (row * K + chunk * 16) and a uniform
+    // offset that walks K.  Rows past the end of the matrix fall outside the
+    // extent and read as zero bytes (fp8 +0.0), which is how tiles that overhang
+    // m or n are handled.
+    uint32_t ld_off[S::LOADS];
+#pragma unroll
+    for (int j = 0; j < S::LOADS; ++j) {
+        const int jj = j < S::A_LOADS ? j : j - S::A_LOADS;
+        const int per = j < S::A_LOADS ? S::A_LOADS : S::B_LOADS;
+        const int row = (wave * per + jj) * RPI + lrow;
+        ld_off[j] = (uint32_t)row * (uint32_t)K + (uint32_t)((lslot ^ tile_swizzle<BK, S::SWZ>(row)) * 16);
+    }
+    const uint32_t ldsA = lds_base + (uint32_t)(wave * S::A_LOADS * RPI * BK);
+    const uint32_t ldsB = lds_base + (uint32_t)(BM * BK + wave * S::B_LOADS * RPI * BK);
+    v4i rsA = {0, 0, 0, 0}, rsB = {0, 0, 0, 0};
+    auto plan_loads = [&](int tile_m, int tile_n) {
+        const int m0 = tile_m * BM, n0 = tile_n * BN;
+        rsA = make_buffer_resource(A + (size_t)m0 * K, (unsigned long long)(M - m0) * (unsigned long long)K);
+        rsB = make_buffer_resource(B + (size_t)n0 * K, (unsigned long long)(N - n0) * (unsigned long long)K);
+    };
+    // load number j (0 .. LOADS-1) of K tile `ktile` into ring slot `stage`
+    auto issue_load = [&](int j, int ktile, int stage) {
+        if (DBG & 1) return;
+        const uint32_t koff = (uint32_t)(ktile * BK);
+        const uint32_t sbase = (uint32_t)(stage * S::STAGE_BYTES);
+        if (j < S::A_LOADS)
+            buffer_load_lds_b128(rsA, ldsA + sbase + (uint32_t)(j * RPI * BK), ld_off[j], koff);
+        else
+            buffer_load_lds_b128(rsB, ldsB + sbase + (uint32_t)((j - S::A_LOADS) * RPI * BK), ld_off[j], koff);
+    };
+    auto issue_all_loads = [&](int ktile, int stage) {
+#pragma unroll
+        for (int j = 0; j < S::LOADS; ++j) issue_load(j, ktile, stage);
+    };
+
+    // All workgroups do the same amount of work per tile, so left alone they all
+    // reach their epilogues together and the C stores of the whole chip hit
+    // memory in one burst while every matrix pipe idles.  Starting the four
+    // phase groups (slot mod 4) a little apart keeps the bursts apart for the
+    // rest of the kernel.  One unit of `stagger` is about 2048 clocks.
+    for (int d = 0; d < (slot & 3) * stagger; ++d) __builtin_amdgcn_s_sleep(32);
+
+    int tile_m = 0, tile_n = 0;
+    bool have = tile_of_round(0, tile_m, tile_n);
+    if (have) {
+        plan_loads(tile_m, tile_n);
+#pragma unroll
+        for (int t = 0; t < STAGES - 1; ++t)
+            if (t < T) issue_all_loads(t, t);
+    }
+
+    for (int r = 0; r < rounds; ++r) {
+        if (!have) {
+            // nothing here this round; still look at the next one
+            have = tile_of_round(r + 1, tile_m, tile_n);
+            if (have) {
+                plan_loads(tile_m, tile_n);
+#pragma unroll
+                for (int t = 0; t < STAGES - 1; ++t)
+                    if (t < T) issue_all_loads(t, t);
+            }
+            continue;
+        }
+        const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+        v16f acc[TM][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.0f;
+
+        // fragment sets: frag[p][0..TM-1] = A blocks, frag[p][TM..TM+TN-1] = B blocks
+        v4i frag[2][TM + TN][2];
+        if (DBG & 4) {
+#pragma unroll
+            for (int p = 0; p < 2; ++p)
+#pragma unroll
+                for (int i = 0; i < TM + TN; ++i)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) frag[p][i][h] = v4i{tid + i, tid * 3 + h, i, p};
+        }
+        // read number q (0 .. NREADS-1) of K step ks of ring slot `stage` into set p.
+        // Order: B0, A0, B1 .. B(TN-1), A1 .. A(TM-1), the order the MFMAs need them.
+        auto issue_read = [&](auto pc, int q, int stage, int ks) {
+            constexpr int P = decltype(pc)::value;
+            if (DBG & 4) return;
+            const int f = q >> 1, h = q & 1;
+            int idx;           // index into frag[P]
+            if (f == 0) idx = TM;
+            else if (f == 1) idx = 0;
+            else if (f <= TN) idx = TM + f - 1;
+            else idx = f - TN;
+            const uint32_t rowbase = idx < TM ? a_base + (uint32_t)(idx * 32 * BK) : b_base + (uint32_t)((idx - TM) * 32 * BK);
+            const uint8_t *p = lds + stage * S::STAGE_BYTES + rowbase + frag_off[ks][h];
+            frag[P][idx][h] = *reinterpret_cast<const v4i *>(p);
+        };
+
+        // K tile 0 must have landed before the first fragment read.  The stores of
+        // the previous tile's epilogue are still in flight and share the counter
+        // with the loads (and may retire out of order with them), so wait for all.
+        wait_vmcnt<0>();
+        __syncthreads();
+        if (STAGES - 1 < T) issue_all_loads(STAGES - 1, STAGES - 1);
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+#pragma unroll
+        for (int q = 0; q < NREADS; ++q) issue_read(I0{}, q, 0, 0);
+
+        // One K step.  P = parity of the global step (which fragment set feeds the
+        // MFMAs), KS = K step inside the K tile, next = a further K tile follows,
+        // load = a K tile STAGES ahead exists and is fetched now (both uniform; the
+        // steady-state loop passes constants so that no branch is left in it).
+        auto kstep = [&](auto pc, auto sc, const bool next, const bool load, int t) {
+            constexpr int P = decltype(pc)::value;
+            constexpr int KS = decltype(sc)::value;
+            using PN = std::integral_constant<int, P ^ 1>;
+            const int stage = t % STAGES;
+            constexpr bool last_ks = (KS + 1 == KSTEPS);
+            int rstage = stage, rks = KS + 1;
+            bool reads = true;
+            if (last_ks) {
+                rstage = (t + 1) % STAGES;
+                rks = 0;
+                reads = next;
+                if (next && !(DBG & 2)) {
+                    // every fragment read of K tile t has been issued; once they have
+                    // returned this wave no longer needs the ring slot
+                    wait_lgkmcnt0();
+                    if (load)
+                        wait_vmcnt<S::LOADS *(STAGES - 2)>();
+                    else
+                        wait_vmcnt<0>();
+                    __syncthreads();
+                }
+            }
+            // reads per MFMA slot and loads per MFMA slot, rounded up
+            constexpr int RD_PER = (NREADS + NMFMA - 1) / NMFMA;
+            constexpr int LD_PER = (S::LOADS + NMFMA - 1) / NMFMA;
+#pragma unroll
+            for (int m = 0; m < NMFMA; ++m) {
+                const int i = m / TN, j = m % TN;
+                acc[i][j] = mfma_32x32x64<BF, AF>(pack8(frag[P][TM + j][0], frag[P][TM + j][1]),
+                                                  pack8(frag[P][i][0], frag[P][i][1]), acc[i][j]);
+                if (last_ks && load) {
+#pragma unroll
+                    for (int u = 0; u < LD_PER; ++u)
+                        if (m * LD_PER + u < S::LOADS) issue_load(m * LD_PER + u, t + STAGES, stage);
+                }
+                if (reads) {
+#pragma unroll
+                    for (int u = 0; u < RD_PER; ++u)
+                        if (m * RD_PER + u < NREADS) issue_read(PN{}, m * RD_PER + u, rstage, rks % KSTEPS);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        // K tiles [0, T-STAGES) fetch ahead, [T-STAGES, T-1) only consume, T-1 is last
+        const int t_load_end = T - STAGES > 0 ? T - STAGES : 0;
+        if (KSTEPS == 2) {
+            int t = 0;
+            for (; t < t_load_end; ++t) {
+                kstep(I0{}, I0{}, true, true, t);
+                kstep(I1{}, I1{}, true, true, t);
+            }
+            for (; t < T; ++t) {
+                kstep(I0{}, I0{}, t + 1 < T, false, t);
+                kstep(I1{}, I1{}, t + 1 < T, false, t);
+            }
+        } else {
+            // K % 128 == 0 makes the number of 64-byte K tiles even: steps go in pairs
+            const int t_pair_end = t_load_end & ~1;
+            int t = 0;
+            for (; t < t_pair_end; t += 2) {
+                kstep(I0{}, I0{}, true, true, t);
+                kstep(I1{}, I0{}, true, true, t + 1);
+            }
+            for (; t < T; t += 2) {
+                kstep(I0{}, I0{}, t + 1 < T, t < t_load_end, t);
+                if (t + 1 < T) kstep(I1{}, I0{}, t + 2 < T, t + 1 < t_load_end, t + 1);
+            }
+        }
+
+        // all waves are done reading LDS for this tile before the ring is reused
+        wait_lgkmcnt0();
+        __syncthreads();
+        int next_m = 0, next_n = 0;
+        have = tile_of_round(r + 1, next_m, next_n);
+        if (have) {
+            plan_loads(next_m, next_n);
+#pragma unroll
+            for (int t = 0; t < STAGES - 1; ++t)
+                if (t < T) issue_all_loads(t, t);
+        }
+
+        // ---- epilogue: registers -> C -------------------------------------------
+        // register q of lane (fi, fg) holds C[row0 + fi][col0 + 8*(q/4) + 4*fg + q%4]
+        const int wrow0 = m0 + wm * (BM / S::WM);
+        const int wcol0 = n0 + wn * (BN / S::WN);
+        const bool full = (m0 + BM <= M) && (n0 + BN <= N) && (N % 4 == 0) &&
+                          (reinterpret_cast<uintptr_t>(C) % 16 == 0);
+        bool skip_store = false;
+        if (DBG & 16) {
+            // tuning: no stores; the data-dependent test keeps the computation alive
+            float chk = 0.0f;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 16; ++q) chk += acc[i][j][q];
+            skip_store = (chk != 12345.678f);
+        }
+        if (skip_store) {
+        } else if (full) {
+            // uniform base per (i, j, q/4); the lane part is one 32-bit offset
+            const uint32_t lane_off = (uint32_t)(fi * N + 4 * fg) * 4u;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; ++q4) {
+                        char *base = reinterpret_cast<char *>(C + (size_t)(wrow0 + i * 32) * N + wcol0 + j * 32 + 8 * q4);
+                        v4f v = {acc[i][j][4 * q4], acc[i][j][4 * q4 + 1], acc[i][j][4 * q4 + 2], acc[i][j][4 * q4 + 3]};
+                        global_store_b128_acc(base, lane_off, v);
+                    }
+        } else {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int row = wrow0 + i * 32 + fi;
+                if (row < M) {
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int q = 0; q < 16; ++q) {
+                            const int col = wcol0 + j * 32 + 8 * (q >> 2) + 4 * fg + (q & 3);
+                            if (col < N) C[(size_t)row * N + col] = acc[i][j][q];
+                        }
+                }
+            }
+        }
+        tile_m = next_m;
+        tile_n = next_n;
+    }
+}
+
+#endif  // FP8GEMM_KERNEL_PTILE_H

@@ -107,6 +107,39 @@ def test_normal_inputs_within_fp32_reordering_bound(pkg, oracle, fa, fb, algo, s
     assert worst < 0.25
 
 
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("shape", [(256, 256, 256), (300, 512, 200), (1000, 1024, 900), (513, 384, 257), (64, 128, 2048)])
+def test_every_tile_variant(pkg, oracle, variant, shape):
+    """Each compiled shape of the tiled kernels (persistent and one-tile-per-workgroup),
+    on shapes that overhang the tile in m and n, for a mixed pairing."""
+    M, K, N = shape
+    rng = np.random.default_rng(zlib.crc32(repr((variant, shape)).encode()))
+    A = random_codes(rng, (M, K), 0)
+    B = random_codes(rng, (N, K), 1)
+    B = np.where(((B >> 2) & 0x1F) > 24, B & 0x83 | 0x3C, B).astype(np.uint8)
+    C = run_gpu(pkg, A, 0, B, 1, algo=ALGOS["tile"], variant=variant)
+    assert_within_bound(oracle, C, A, 0, B, 1, hw_term=True)
+
+
+@pytest.mark.parametrize("stages", [2, 4])
+@pytest.mark.parametrize("fa,fb", PAIRS)
+def test_entry_points_stage2_stage4(pkg, oracle, fa, fb, stages):
+    """The eight per-precision entry points (GEMM / GEMM4 of the reference), default stream."""
+    import torch
+    M, K, N = 512, 1024, 768
+    A = pkg.fill((M, K), fa, seed=3, dist="normal", sigma=4.0)
+    B = pkg.fill((N, K), fb, seed=4, dist="normal", sigma=4.0)
+    dt = {0: torch.float8_e4m3fn, 1: torch.float8_e5m2}
+    dA = torch.from_numpy(A).cuda().view(dt[fa])
+    dB = torch.from_numpy(B).cuda().view(dt[fb])
+    out = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    fn = pkg.GEMM if stages == 2 else pkg.GEMM4
+    assert fn(M, K, N, dA, dB, out) == 0
+    torch.cuda.synchronize()
+    assert_within_bound(oracle, out.cpu().numpy(), A, fa, B, fb)
+
+
 @pytest.mark.parametrize("fa,fb", PAIRS)
 @pytest.mark.parametrize("algo", ["direct", "tile", "skinny"])
 def test_decode_through_mfma_is_bit_exact(pkg, oracle, fa, fb, algo):
