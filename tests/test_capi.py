@@ -1,0 +1,100 @@
+"""Host side of the C ABI: the library loads, exports every declared symbol, validates its
+arguments before touching the GPU, and generates reproducible operands."""
+import ctypes
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+
+def declared_symbols(header):
+    text = open(header).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fp8gemm_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_symbol_of_the_header(pkg):
+    L = pkg.lib()
+    names = declared_symbols(pkg.HEADER_PATH)
+    assert len(names) >= 20 and all(n in names for n in pkg.ENTRY_POINTS)
+    for n in names:
+        assert hasattr(L, n), "missing export " + n
+    nm = subprocess.run(["nm", "-D", "--defined-only", pkg.LIB_PATH], capture_output=True, text=True).stdout
+    for n in names:
+        assert re.search(r"\bT %s\b" % n, nm), "not a defined text symbol: " + n
+
+
+def test_argument_validation_needs_no_gpu(pkg):
+    L = pkg.lib()
+    INVALID = 1      # hipErrorInvalidValue
+    ok_ptr = ctypes.c_void_p(0x1000)
+    assert L.fp8gemm_launch(0, 128, 128, ok_ptr, 0, ok_ptr, 0, ok_ptr, 2, None) == INVALID
+    assert L.fp8gemm_launch(128, -1, 128, ok_ptr, 0, ok_ptr, 0, ok_ptr, 2, None) == INVALID
+    assert L.fp8gemm_launch(128, 128, 128, None, 0, ok_ptr, 0, ok_ptr, 2, None) == INVALID
+    assert L.fp8gemm_launch(128, 128, 128, ok_ptr, 0, None, 0, ok_ptr, 2, None) == INVALID
+    assert L.fp8gemm_launch(128, 128, 128, ok_ptr, 0, ok_ptr, 0, None, 2, None) == INVALID
+    assert L.fp8gemm_launch(128, 128, 128, ok_ptr, 2, ok_ptr, 0, ok_ptr, 2, None) == INVALID
+    assert L.fp8gemm_launch(128, 128, 128, ok_ptr, 0, ok_ptr, -1, ok_ptr, 2, None) == INVALID
+    assert L.fp8gemm_launch(128, 128, 128, ok_ptr, 0, ok_ptr, 0, ok_ptr, 3, None) == INVALID
+    assert L.fp8gemm_launch_algo(128, 128, 128, ok_ptr, 0, ok_ptr, 0, ok_ptr, 2, 9, None) == INVALID
+    for name in pkg.ENTRY_POINTS:
+        assert getattr(L, name)(128, 128, 128, None, None, None) == INVALID
+        assert getattr(L, name)(128, 0, 128, ok_ptr, ok_ptr, ok_ptr) == INVALID
+    assert b"invalid" in L.fp8gemm_error_string(INVALID).lower()
+    assert L.fp8gemm_version() >= 100
+
+
+def test_kernel_selection_is_pure_host_logic(pkg):
+    L = pkg.lib()
+    assert L.fp8gemm_select_algo(8192, 8192, 8192) == pkg.ALGO_TILE
+    assert L.fp8gemm_select_algo(16, 8192, 28672) == pkg.ALGO_SKINNY
+    assert L.fp8gemm_select_algo(1, 28672, 8192) == pkg.ALGO_SKINNY
+    assert L.fp8gemm_select_algo(64, 8192, 10240) == pkg.ALGO_SKINNY
+    assert L.fp8gemm_select_algo(256, 8192, 28672) == pkg.ALGO_TILE
+    assert L.fp8gemm_select_algo(100, 100, 100) == pkg.ALGO_DIRECT       # k not a multiple of 128
+    assert L.fp8gemm_select_algo(16, 100, 64) == pkg.ALGO_DIRECT
+    assert L.fp8gemm_select_algo(0, 1, 1) == -1
+    assert L.fp8gemm_num_variants(pkg.ALGO_TILE) >= 2 and L.fp8gemm_num_variants(pkg.ALGO_SKINNY) >= 1
+    assert L.fp8gemm_scratch_bytes(8192, 8192, 8192) == 0
+    s = L.fp8gemm_scratch_bytes(16, 28672, 8192)
+    assert s % (16 * 8192 * 4) == 0        # whole partial-sum planes, or none
+
+
+def test_generators_are_reproducible_and_counter_based(pkg):
+    for dist in ("uniform", "normal", "weights", "loguniform"):
+        for fmt in (0, 1):
+            a = pkg.fill((300, 70), fmt, seed=42, dist=dist)
+            b = pkg.fill((300, 70), fmt, seed=42, dist=dist)
+            c = pkg.fill((300, 70), fmt, seed=43, dist=dist)
+            assert np.array_equal(a, b) and not np.array_equal(a, c)
+            if dist != "weights":     # element i depends on (seed, i) only: a prefix is a prefix
+                assert np.array_equal(pkg.fill((100, 70), fmt, seed=42, dist=dist).ravel(), a.ravel()[:7000])
+
+
+def test_generator_distributions(pkg, oracle):
+    n = 400_000
+    for fmt, top, lo in ((0, 448.0, 2.0 ** -9), (1, 57344.0, 2.0 ** -16)):
+        x = oracle.decode(pkg.fill((n,), fmt, seed=7, dist="normal"), fmt)
+        assert abs(x.mean()) < 0.01 and abs(x.std() - 1.0) < 0.03
+        u = oracle.decode(pkg.fill((n,), fmt, seed=7, dist="uniform"), fmt)
+        assert u.min() >= -1.0 and u.max() <= 1.0 and abs(u.mean()) < 0.01 and abs(u.std() - 3 ** -0.5) < 0.02
+        w = oracle.decode(pkg.fill((n,), fmt, seed=7, dist="weights", sigma=0.02), fmt)
+        assert np.abs(w).max() == top and abs(w.mean()) < top * 0.01
+        g_codes = pkg.fill((n,), fmt, seed=7, dist="loguniform")
+        g = oracle.decode(g_codes, fmt)
+        assert np.isfinite(g).all() and np.abs(g).max() <= top
+        nz = np.abs(g[g != 0])
+        assert nz.min() == lo and nz.max() >= top / 2          # whole exponent range, subnormals included
+        assert 0.45 < (g < 0).mean() < 0.55
+        e = np.floor(np.log2(nz))
+        counts = np.bincount((e - e.min()).astype(int))
+        assert counts.min() > 0.5 * counts.mean()               # roughly flat over binades
+
+
+def test_python_entry_points_refuse_host_tensors(pkg):
+    import torch
+    a = torch.zeros((16, 128), dtype=torch.uint8)
+    with pytest.raises(pkg.Fp8GemmError):
+        pkg.gemm(a, a, a_fmt=0, b_fmt=0)
