@@ -24,8 +24,8 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E peak, GB/s
 
 # HBM bytes moved by one 8192^3 launch of the tiled kernel, from rocprofv3
 # FETCH_SIZE / WRITE_SIZE counter runs scaled by the reading of a plain copy
-# kernel of known size (summary under profiles/).  None until measured.
-TRAFFIC_BYTES_8192 = None
+# kernel of known size (summary under profiles/).
+TRAFFIC_BYTES_8192 = (2 * 394178 + 308809) * 1024   # FETCH_SIZE x 2.0 (copy-kernel scale) + WRITE_SIZE x 1.0, KiB -> bytes
 
 
 def load_package():
@@ -68,6 +68,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host CPU leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy, the known-size kernel that FETCH_SIZE / WRITE_SIZE "
+                         "counter readings are scaled by when this script runs under rocprofv3 --pmc")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU: the FP8 GEMM path has no multi-GPU part in this build "
@@ -80,6 +83,14 @@ def main():
     pkg = load_package()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(3)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)          # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---------------------------------------------------------------- square, compute-bound
     M = N = K = 8192

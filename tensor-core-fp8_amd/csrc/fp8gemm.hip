@@ -223,33 +223,33 @@ bool skinny_ok(int m, int k, int n)
     return m <= 64 && n % 16 == 0 && k % 256 == 0;
 }
 
-// Picks columns per wave, LDS shape and split-K factor so that the number of
-// independent streams is close to a multiple of the CU count and every stream
-// is long enough to amortise its start-up.
+// Picks columns per wave, LDS shape and split-K factor.  Measured on MI355X:
+// the HBM pipe is fullest with about two fat streams per CU (each with a deep
+// LDS ring), not with many thin ones, and a split-K pass costs a few percent.
+// So: aim at 512 streams, prefer no split, then wider streams.
 SkinnyPlan plan_skinny(int m, int k, int n)
 {
     SkinnyPlan p;
     p.mt = (m + 15) / 16;
-    p.variant = 1;
-    int tn = (p.mt >= 3) ? 4 : p.mt;              // keep A traffic <= B traffic
-    while (tn > 1 && n % (16 * tn) != 0) tn /= 2;
-    p.tn = tn;
-    const int groups = n / (16 * tn);
+    const int tn_min = (p.mt >= 3) ? 2 : 1;       // keep the re-read of A below the read of B
     const int ksteps = k / 256;
-    constexpr int kCUs = 256;
-    int best = 1;
-    double best_score = -1.0;
-    for (int s = 1; s <= 16; ++s) {
-        if (ksteps % s != 0 || ksteps / s < 4) continue;
-        const long units = (long)groups * s;
-        const long rounds = (units + kCUs - 1) / kCUs;
-        double eff = (double)units / (double)(rounds * kCUs);   // tail balance
-        if (rounds < 2) eff *= 0.5 + 0.25 * rounds;             // too few streams per CU
-        if (rounds > 8) eff *= 0.9;                             // more than LDS can hold at once
-        const double score = eff - 0.03 * (s - 1);              // reduction pass is not free
-        if (score > best_score) { best_score = score; best = s; }
+    int best_tn = 1, best_split = 1;
+    long best_cost = -1;
+    for (int tn = 4; tn >= 1; tn /= 2) {
+        if (n % (16 * tn) != 0) continue;
+        if (tn < tn_min && n % (16 * tn_min) == 0) continue;
+        for (int s = 1; s <= 16; s *= 2) {
+            if (ksteps % s != 0 || ksteps / s < 4) continue;
+            const long streams = (long)(n / (16 * tn)) * s;
+            long cost = (streams > 512 ? streams - 512 : 512 - streams) * 4;   // distance from the sweet spot
+            cost += (s - 1) * 96;                                               // reduction pass, partial-sum traffic
+            cost += (4 - tn) * 8;                                               // A is re-read once per stream
+            if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_tn = tn; best_split = s; }
+        }
     }
-    p.nsplit = best;
+    p.tn = best_tn;
+    p.nsplit = best_split;
+    p.variant = (best_tn == 4) ? 0 : 1;           // 128-byte K steps for wide streams, 256 otherwise
     return p;
 }
 
