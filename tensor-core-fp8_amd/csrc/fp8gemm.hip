@@ -19,7 +19,6 @@ namespace {
 
 constexpr int kVersion = 100;
 constexpr int kMaxDevices = 64;
-constexpr int kDefaultStagger = 1;    // units of ~2048 clocks between phase groups of the persistent kernel
 
 // ------------------------------------------------------------------ variants
 // Tiled kernel shapes: <BM, BN, BK, waves_m, waves_n, stages, swizzle>.
@@ -134,13 +133,11 @@ hipError_t launch_ptile_shape(int m, int k, int n, const uint8_t *a, const uint8
     const int nb = ((tiles_m + GM - 1) / GM) * ((tiles_n + GN - 1) / GN);
     const int rounds = (nb + 7) / 8;
     const int grid = 8 * GM * GN;
-    // phase stagger only pays when a workgroup has several tiles to write
-    const int stagger = rounds >= 2 ? kDefaultStagger : 0;
     auto kernel = gemm_ptile_kernel<S, AF, BF>;
-    hipError_t e = allow_lds(kernel, S::LDS_BYTES);
+    hipError_t e = allow_lds(kernel, S::PTILE_LDS_BYTES);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(S::THREADS), S::LDS_BYTES, stream,
-                       m, k, n, a, b, out, tiles_m, tiles_n, GM, GN, rounds, stagger);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(S::THREADS), S::PTILE_LDS_BYTES, stream,
+                       m, k, n, a, b, out, tiles_m, tiles_n, GM, GN, rounds);
     return hipGetLastError();
 }
 

@@ -48,12 +48,12 @@ __device__ __forceinline__ void buffer_load_lds_b128(v4i rsrc, uint32_t lds_addr
                  : "m0");
 }
 
-// 16-byte-per-lane store whose data operand stays in accumulation registers
-// (the MFMA results live there; a store can read them directly, a copy to
-// ordinary vector registers first would need 256 more registers per lane).
-__device__ __forceinline__ void global_store_b128_acc(void *uniform_base, uint32_t lane_off, v4f data)
+// 16-byte-per-lane LDS store whose data operand stays in accumulation registers
+// (the MFMA results live there; copying all of them to ordinary vector registers
+// first would need 256 more registers per lane).
+__device__ __forceinline__ void lds_store_b128_acc(uint32_t lds_addr, v4f data)
 {
-    asm volatile("global_store_dwordx4 %0, %1, %2" : : "v"(lane_off), "a"(data), "s"(uniform_base) : "memory");
+    asm volatile("ds_write_b128 %0, %1" : : "v"(lds_addr), "a"(data) : "memory");
 }
 
 __device__ __forceinline__ v4i make_buffer_resource(const void *base, unsigned long long bytes)
@@ -76,7 +76,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                                                                  const uint8_t *__restrict__ B,
                                                                  float *__restrict__ C,
                                                                  int tiles_m, int tiles_n, int GM, int GN,
-                                                                 int rounds, int stagger)
+                                                                 int rounds)
 {
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, CH = S::CH, RPI = S::RPI;
     constexpr int STAGES = S::STAGES, TM = S::TM, TN = S::TN, KSTEPS = S::KSTEPS;
@@ -158,13 +158,6 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
 #pragma unroll
         for (int j = 0; j < S::LOADS; ++j) issue_load(j, ktile, stage);
     };
-
-    // All workgroups do the same amount of work per tile, so left alone they all
-    // reach their epilogues together and the C stores of the whole chip hit
-    // memory in one burst while every matrix pipe idles.  Starting the four
-    // phase groups (slot mod 4) a little apart keeps the bursts apart for the
-    // rest of the kernel.  One unit of `stagger` is about 2048 clocks.
-    for (int d = 0; d < (slot & 3) * stagger; ++d) __builtin_amdgcn_s_sleep(32);
 
     int tile_m = 0, tile_n = 0;
     bool have = tile_of_round(0, tile_m, tile_n);
@@ -340,18 +333,35 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         }
         if (skip_store) {
         } else if (full) {
-            // uniform base per (i, j, q/4); the lane part is one 32-bit offset
-            const uint32_t lane_off = (uint32_t)(fi * N + 4 * fg) * 4u;
+            // Each wave transposes its results through a private strip of LDS (the part of
+            // the ring the next tile's first loads do not use, plus the LDS above the ring)
+            // so that every store instruction writes whole contiguous row segments of C:
+            // a CU drains full-line stores about three times faster than 32-byte pieces.
+            constexpr int EP = S::EP_COLS;                       // columns staged at a time
+            constexpr int ROWB = EP * 4 + 16;                    // padded row: conflict-free both ways
+            constexpr int LPR = EP / 4;                          // lanes per row when reading back
+            constexpr int RPI_ST = 64 / LPR;                     // rows per store instruction
+            uint8_t *stg = lds + S::EP_OFFSET + wave * (32 * ROWB);
+            const uint32_t stg_addr = lds_base + (uint32_t)(S::EP_OFFSET + wave * (32 * ROWB));
+            const int rl = lane / LPR, cl = lane % LPR;
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
+                for (int c0 = 0; c0 < TN * 32; c0 += EP) {
 #pragma unroll
-                    for (int q4 = 0; q4 < 4; ++q4) {
-                        char *base = reinterpret_cast<char *>(C + (size_t)(wrow0 + i * 32) * N + wcol0 + j * 32 + 8 * q4);
-                        v4f v = {acc[i][j][4 * q4], acc[i][j][4 * q4 + 1], acc[i][j][4 * q4 + 2], acc[i][j][4 * q4 + 3]};
-                        global_store_b128_acc(base, lane_off, v);
+                    for (int j = c0 / 32; j < (c0 + EP) / 32; ++j)
+#pragma unroll
+                        for (int q4 = 0; q4 < 4; ++q4) {
+                            v4f v = {acc[i][j][4 * q4], acc[i][j][4 * q4 + 1], acc[i][j][4 * q4 + 2], acc[i][j][4 * q4 + 3]};
+                            lds_store_b128_acc(stg_addr + (uint32_t)(fi * ROWB + (j * 32 - c0 + 8 * q4 + 4 * fg) * 4), v);
+                        }
+#pragma unroll
+                    for (int r0 = 0; r0 < 32; r0 += RPI_ST) {
+                        const v4f v = *reinterpret_cast<const v4f *>(stg + (r0 + rl) * ROWB + cl * 16);
+                        float *dst = C + (size_t)(wrow0 + i * 32 + r0 + rl) * N + wcol0 + c0 + cl * 4;
+                        *reinterpret_cast<v4f *>(dst) = v;
                     }
+                }
         } else {
 #pragma unroll
             for (int i = 0; i < TM; ++i) {

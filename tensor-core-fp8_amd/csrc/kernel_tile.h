@@ -56,6 +56,15 @@ struct TileShape {
     static constexpr int TM = BM / WM / 32;       // 32x32 MFMA tiles per wave, M direction
     static constexpr int TN = BN / WN / 32;
     static constexpr int KSTEPS = BK / 64;
+    // epilogue staging of the persistent kernel: LDS not used by the next tile's first
+    // STAGES-1 K tiles (the last ring slot and whatever lies between the ring and 160 KiB)
+    static constexpr int LDS_MAX = 160 * 1024;
+    static constexpr int EP_OFFSET = STAGE_BYTES * (STAGES - 1);
+    static constexpr int EP_WIDE = BN / WN;                                       // all columns of a wave at once
+    static constexpr int EP_COLS = (NW * 32 * (EP_WIDE * 4 + 16) <= LDS_MAX - EP_OFFSET) ? EP_WIDE : EP_WIDE / 2;
+    static constexpr int EP_BYTES = NW * 32 * (EP_COLS * 4 + 16);
+    static constexpr int PTILE_LDS_BYTES = (EP_OFFSET + EP_BYTES > LDS_BYTES) ? EP_OFFSET + EP_BYTES : LDS_BYTES;
+    static_assert(EP_OFFSET + EP_BYTES <= LDS_MAX, "epilogue staging does not fit");
     static_assert(BM % (RPI * NW) == 0 && BN % (RPI * NW) == 0, "tile rows must split over waves");
     static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be whole MFMA tiles");
     static_assert(LOADS * (STAGES - 1) < 64, "vmcnt cannot count that many loads");
