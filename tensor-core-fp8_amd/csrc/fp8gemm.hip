@@ -27,7 +27,9 @@ using TileP4 = TileShape<256, 256, 64, 2, 2, 4, 2>;   // persistent, 4 x 32 KiB 
 using TileP8 = TileShape<256, 256, 128, 2, 4, 2, 3>;  // persistent, 8 waves, 128x64 per wave
 using TileS2 = TileShape<128, 128, 128, 2, 2, 2, 3>;  // one tile per workgroup, for small problems
 using TileS4 = TileShape<128, 128, 128, 2, 2, 4, 3>;
-constexpr int kNumTileVariants = 5;               // 0 P2, 1 P4, 2 P8, 3 S2, 4 S4
+using TileH2 = TileShape<128, 256, 128, 2, 2, 2, 3>;  // persistent, half-height tile: more tiles for short-m problems
+using TileQ2 = TileShape<128, 128, 128, 2, 2, 2, 3>;  // persistent, quarter tile
+constexpr int kNumTileVariants = 7;               // 0 P2, 1 P4, 2 P8, 3 S2, 4 S4, 5 H2, 6 Q2
 
 // Skinny kernel shapes: <MT, TN, BK, stages>.
 template <int MT, int TN>
@@ -127,9 +129,11 @@ hipError_t launch_ptile_shape(int m, int k, int n, const uint8_t *a, const uint8
     if (k % S::BK != 0) return hipErrorInvalidValue;
     const int tiles_m = (m + S::BM - 1) / S::BM;
     const int tiles_n = (n + S::BN - 1) / S::BN;
-    int GM = 4, GN = 8;                       // 32 tiles = the 32 CUs of one XCD
-    if (tiles_m < GM) { GM = tiles_m; }
-    if (tiles_n < GN) { GN = tiles_n; }
+    // 32 tiles = the 32 CUs of one XCD; 4 x 8 when the grid of tiles allows, else as
+    // close to 32 as it gets
+    int GM = tiles_m < 4 ? tiles_m : 4;
+    int GN = tiles_n < 32 / GM ? tiles_n : 32 / GM;
+    GM = tiles_m < 32 / GN ? tiles_m : 32 / GN;
     const int nb = ((tiles_m + GM - 1) / GM) * ((tiles_n + GN - 1) / GN);
     const int rounds = (nb + 7) / 8;
     const int grid = 8 * GM * GN;
@@ -151,6 +155,8 @@ hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, 
     case 2: return launch_ptile_shape<TileP8, AF, BF>(m, k, n, a, b, out, stream);
     case 3: return launch_tile_shape<TileS2, AF, BF>(m, k, n, a, b, out, stream);
     case 4: return launch_tile_shape<TileS4, AF, BF>(m, k, n, a, b, out, stream);
+    case 5: return launch_ptile_shape<TileH2, AF, BF>(m, k, n, a, b, out, stream);
+    case 6: return launch_ptile_shape<TileQ2, AF, BF>(m, k, n, a, b, out, stream);
     default: return hipErrorInvalidValue;
     }
 }

@@ -107,7 +107,7 @@ def test_normal_inputs_within_fp32_reordering_bound(pkg, oracle, fa, fb, algo, s
     assert worst < 0.25
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("shape", [(256, 256, 256), (300, 512, 200), (1000, 1024, 900), (513, 384, 257), (64, 128, 2048)])
 def test_every_tile_variant(pkg, oracle, variant, shape):
     """Each compiled shape of the tiled kernels (persistent and one-tile-per-workgroup),
