@@ -52,6 +52,12 @@ def lib():
         raise Fp8GemmError(
             "libfp8gemm.so is not built (%s); run __graft_entry__.build() or "
             "`make -C tensor-core-fp8_amd/GEMM lib`" % LIB_PATH)
+    # torch ships its own copy of the HIP runtime; when both end up in one process the
+    # copy loaded first is the one that owns the device, so let torch load first
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     L = ctypes.CDLL(LIB_PATH)
     vp, ci = ctypes.c_void_p, ctypes.c_int
     for name in ENTRY_POINTS:

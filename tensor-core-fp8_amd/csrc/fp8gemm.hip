@@ -313,6 +313,9 @@ int launch_checked(int m, int k, int n, const void *a, int a_fmt, const void *b,
     const uint8_t *pa = static_cast<const uint8_t *>(a);
     const uint8_t *pb = static_cast<const uint8_t *>(b);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    // the launch status is read back with hipGetLastError(); drop whatever an earlier,
+    // unrelated runtime call of this thread may have left there
+    (void)hipGetLastError();
     hipError_t e;
     if (a_fmt == FP8GEMM_E4M3 && b_fmt == FP8GEMM_E4M3)
         e = dispatch<0, 0>(m, k, n, pa, pb, out, stages, algo, variant, nsplit, s);
