@@ -40,7 +40,11 @@ template <int MT, int TN>
 using SkinnyV2 = SkinnyShape<MT, TN, 128, 8>;
 template <int MT, int TN>
 using SkinnyV3 = SkinnyShape<MT, TN, 256, 6>;
-constexpr int kNumSkinnyVariants = 4;
+template <int MT, int TN>
+using SkinnyV4 = SkinnyShape<MT, TN, 512, 4, 80 * 1024>;
+template <int MT, int TN>
+using SkinnyV5 = SkinnyShape<MT, TN, 1024, 3, 80 * 1024>;
+constexpr int kNumSkinnyVariants = 6;
 
 struct Scratch {
     void *ptr = nullptr;
@@ -166,7 +170,7 @@ struct SkinnyPlan {
     int mt, tn, variant, nsplit;
 };
 
-template <class S, int AF, int BF>
+template <class S, int AF, int BF, int DBG = 0>
 hipError_t launch_skinny_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
                                int nsplit, hipStream_t stream)
 {
@@ -181,7 +185,7 @@ hipError_t launch_skinny_shape(int m, int k, int n, const uint8_t *a, const uint
         if (e != hipSuccess) return e;
         dst = static_cast<float *>(ws);
     }
-    auto kernel = gemm_skinny_kernel<S, AF, BF>;
+    auto kernel = gemm_skinny_kernel<S, AF, BF, DBG>;
     hipError_t e = allow_lds(kernel, S::LDS_BYTES);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3((unsigned)(ngroups * nsplit)), dim3(64), S::LDS_BYTES, stream,
@@ -217,42 +221,46 @@ hipError_t launch_skinny(int m, int k, int n, const uint8_t *a, const uint8_t *b
     case 1: return launch_skinny_mt<SkinnyV1, AF, BF>(m, k, n, a, b, out, p, stream);
     case 2: return launch_skinny_mt<SkinnyV2, AF, BF>(m, k, n, a, b, out, p, stream);
     case 3: return launch_skinny_mt<SkinnyV3, AF, BF>(m, k, n, a, b, out, p, stream);
+    case 4: return launch_skinny_mt<SkinnyV4, AF, BF>(m, k, n, a, b, out, p, stream);
+    case 5: return launch_skinny_mt<SkinnyV5, AF, BF>(m, k, n, a, b, out, p, stream);
+#ifdef FP8GEMM_TUNING
+    case 10: return launch_skinny_shape<SkinnyV0<1, 4>, AF, BF, 1>(m, k, n, a, b, out, p.nsplit, stream);
+    case 11: return launch_skinny_shape<SkinnyV0<1, 4>, AF, BF, 2>(m, k, n, a, b, out, p.nsplit, stream);
+    case 12: return launch_skinny_shape<SkinnyV0<1, 4>, AF, BF, 3>(m, k, n, a, b, out, p.nsplit, stream);
+    case 13: return launch_skinny_shape<SkinnyV1<1, 1>, AF, BF, 3>(m, k, n, a, b, out, p.nsplit, stream);
+    case 14: return launch_skinny_shape<SkinnyV5<1, 1>, AF, BF, 3>(m, k, n, a, b, out, p.nsplit, stream);
+#endif
     default: return hipErrorInvalidValue;
     }
 }
 
 bool skinny_ok(int m, int k, int n)
 {
-    return m <= 64 && n % 16 == 0 && k % 256 == 0;
+    return m <= 64 && n % 16 == 0 && k % 128 == 0;
 }
 
-// Picks columns per wave, LDS shape and split-K factor.  Measured on MI355X:
-// the HBM pipe is fullest with about two fat streams per CU (each with a deep
-// LDS ring), not with many thin ones, and a split-K pass costs a few percent.
-// So: aim at 512 streams, prefer no split, then wider streams.
+// Picks columns per wave, LDS shape and split-K factor.  Measured on MI355X with
+// operands that are cold in every cache: the HBM pipe is fullest with one to two
+// fat streams per CU (256..512 streams, each with a deep LDS ring) rather than many
+// thin ones; a split-K pass costs 10 % and more, so it is used only when the
+// columns alone give too few streams; long K steps (512 bytes per row and load
+// group) help a little.
 SkinnyPlan plan_skinny(int m, int k, int n)
 {
     SkinnyPlan p;
     p.mt = (m + 15) / 16;
     const int tn_min = (p.mt >= 3) ? 2 : 1;       // keep the re-read of A below the read of B
-    const int ksteps = k / 256;
-    int best_tn = 1, best_split = 1;
-    long best_cost = -1;
-    for (int tn = 4; tn >= 1; tn /= 2) {
-        if (n % (16 * tn) != 0) continue;
-        if (tn < tn_min && n % (16 * tn_min) == 0) continue;
-        for (int s = 1; s <= 16; s *= 2) {
-            if (ksteps % s != 0 || ksteps / s < 4) continue;
-            const long streams = (long)(n / (16 * tn)) * s;
-            long cost = (streams > 512 ? streams - 512 : 512 - streams) * 4;   // distance from the sweet spot
-            cost += (s - 1) * 96;                                               // reduction pass, partial-sum traffic
-            cost += (4 - tn) * 8;                                               // A is re-read once per stream
-            if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_tn = tn; best_split = s; }
-        }
-    }
-    p.tn = best_tn;
-    p.nsplit = best_split;
-    p.variant = (best_tn == 4) ? 0 : 1;           // 128-byte K steps for wide streams, 256 otherwise
+    int tn = 4;
+    while (tn > 1 && (n % (16 * tn) != 0 || (n / (16 * tn) < 256 && tn > tn_min))) tn /= 2;
+    while (n % (16 * tn) != 0) tn /= 2;           // n % 16 == 0 is guaranteed by the caller
+    const int ksteps = k / 128;
+    int split = 1;
+    while ((long)(n / (16 * tn)) * split < 192 && split < 16 && ksteps % (2 * split) == 0 && ksteps / (2 * split) >= 8)
+        split *= 2;
+    p.tn = tn;
+    p.nsplit = split;
+    const int kchunk = k / split;
+    p.variant = (kchunk % 512 == 0) ? 4 : (kchunk % 256 == 0) ? 1 : 0;
     return p;
 }
 

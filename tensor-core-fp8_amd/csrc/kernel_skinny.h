@@ -24,20 +24,31 @@
 
 constexpr int skinny_min3(int a, int b, int c) { return a < b ? (a < c ? a : c) : (b < c ? b : c); }
 
-// STAGES_ is the wanted ring depth; it is cut back so that the loads in flight
-// stay countable by vmcnt (6 bits) and the ring stays within LDS_CAP_ bytes.
+// Largest K step <= bk (halving) for which two ring slots of (mt+tn)*16 rows fit in
+// `cap` bytes of LDS and one slot's loads stay countable by vmcnt.
+constexpr int skinny_fit_bk(int mt, int tn, int bk, int cap)
+{
+    while (bk > 128 && ((mt + tn) * 16 * bk * 2 > cap || (mt + tn) * 16 * bk / 1024 > 31)) bk /= 2;
+    return bk;
+}
+
+// BK_ is the wanted K step and STAGES_ the wanted ring depth; both are cut back so
+// that the ring stays within LDS_CAP_ bytes and the loads in flight stay countable
+// by vmcnt (6 bits).
 template <int MT_, int TN_, int BK_, int STAGES_, int LDS_CAP_ = 64 * 1024>
 struct SkinnyShape {
-    static constexpr int MT = MT_, TN = TN_, BK = BK_;
-    static constexpr int STAGES = skinny_min3(STAGES_, 63 / ((MT_ + TN_) * 16 / (64 / (BK_ / 16))) + 1,
-                                              LDS_CAP_ / ((MT_ + TN_) * 16 * BK_));
+    static constexpr int MT = MT_, TN = TN_;
+    static constexpr int BK = skinny_fit_bk(MT_, TN_, BK_, LDS_CAP_);
+    static constexpr int STAGES = skinny_min3(STAGES_, 63 / ((MT_ + TN_) * 16 * BK / 1024) + 1,
+                                              LDS_CAP_ / ((MT_ + TN_) * 16 * BK));
     static constexpr int MP = MT * 16;            // padded rows of A
     static constexpr int NP = TN * 16;            // columns of C per wave
     static constexpr int CH = BK / 16;            // 16-byte chunks per row
-    static constexpr int RPI = 64 / CH;           // rows per wave-wide load
+    static constexpr int RPI = 64 / CH > 0 ? 64 / CH : 1;   // rows per wave-wide load
+    static constexpr int LPR = CH / 64 > 0 ? CH / 64 : 1;   // wave-wide loads per row (BK = 1024: 1)
     static constexpr int ROWS = MP + NP;
-    static constexpr int LOADS = ROWS / RPI;      // direct loads per K step
-    static constexpr int A_LOADS = MP / RPI;
+    static constexpr int LOADS = ROWS * BK / 1024;          // direct loads per K step
+    static constexpr int A_LOADS = MP * BK / 1024;
     static constexpr int STAGE_BYTES = ROWS * BK;
     static constexpr int LDS_BYTES = STAGE_BYTES * STAGES;
     static constexpr int KSTEPS = BK / 128;       // MFMA K steps per stage
@@ -57,7 +68,9 @@ __device__ __forceinline__ int skinny_swizzle(int row)
     return ((row & 7) ^ ((row >> 3) & 1));
 }
 
-template <class S, int AF, int BF>
+// DBG (tuning builds only, wrong results on purpose): bit 0 drops the loads of A,
+// bit 1 the fragment reads and MFMAs.
+template <class S, int AF, int BF, int DBG = 0>
 __global__ __launch_bounds__(64) void gemm_skinny_kernel(int M, int K, int N,
                                                          const uint8_t *__restrict__ A,
                                                          const uint8_t *__restrict__ B,
@@ -89,9 +102,16 @@ __global__ __launch_bounds__(64) void gemm_skinny_kernel(int M, int K, int N,
             src[j] = B + (size_t)(n0 + row - MP) * K + kbeg + chunk * 16;
         }
     }
-    auto issue_loads = [&](int t, int stage) {
+    // Every stream starts its K walk at a different K step (and wraps around): streams
+    // that start together would otherwise sweep the same address bits -- the same HBM
+    // channels -- at the same time.  The rotation only reorders the fp32 sum.
+    const int T = kchunk / BK;
+    const int t0 = (int)(((unsigned)group * 2654435761u >> 8) % (unsigned)T);
+    auto issue_loads = [&](int tt, int stage) {
+        int t = tt + t0;
+        t = t >= T ? t - T : t;
 #pragma unroll
-        for (int j = 0; j < S::LOADS; ++j)
+        for (int j = (DBG & 1) ? S::A_LOADS : 0; j < S::LOADS; ++j)
             __builtin_amdgcn_global_load_lds((const GLOBAL_AS void *)(src[j] + (size_t)t * BK),
                                              (LDS_AS void *)(lds + stage * S::STAGE_BYTES + j * RPI * BK),
                                              16, 0, 0);
@@ -114,7 +134,6 @@ __global__ __launch_bounds__(64) void gemm_skinny_kernel(int M, int K, int N,
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
-    const int T = kchunk / BK;
 #pragma unroll
     for (int t = 0; t < STAGES - 1; ++t)
         if (t < T) issue_loads(t, t);
@@ -123,13 +142,13 @@ __global__ __launch_bounds__(64) void gemm_skinny_kernel(int M, int K, int N,
         // refill the stage consumed one step ago, then wait for stage t
         if (t + STAGES - 1 < T) {
             issue_loads(t + STAGES - 1, (t + STAGES - 1) % STAGES);
-            wait_vmcnt<S::LOADS *(STAGES - 1)>();
+            wait_vmcnt<((DBG & 1) ? S::LOADS - S::A_LOADS : S::LOADS) * (STAGES - 1)>();
         } else {
             wait_vmcnt<0>();
         }
         const uint8_t *st = lds + (t % STAGES) * S::STAGE_BYTES;
 #pragma unroll
-        for (int s = 0; s < S::KSTEPS; ++s) {
+        for (int s = 0; s < ((DBG & 2) ? 0 : S::KSTEPS); ++s) {
             v8i af[MT], bf[TN];
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
