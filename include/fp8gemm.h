@@ -71,8 +71,11 @@ int fp8gemm_launch_algo(int m, int k, int n, const void *a, int a_fmt, const voi
  * Tuning hook with no counterpart in the reference: forces a kernel family
  * and one of its compiled shape variants (0 .. fp8gemm_num_variants(algo)-1,
  * -1 = the default for the shape).  For FP8GEMM_ALGO_SKINNY, variant may add
- * 16 * columns-per-wave/16 to override the planned column count per wave, and
- * split_k > 0 overrides the planned split-K factor.
+ * 16 * columns-per-wave/16 to override the planned column count per wave; for
+ * FP8GEMM_ALGO_TILE it may add 16 * (1 + r) to force the K-walk rotation mode
+ * r (0 none, 1 per tile column, 2 per block of tiles).  split_k > 0 overrides
+ * the planned number of K slices (skinny kernel and persistent tiled kernels);
+ * a forced tile variant runs unsplit unless split_k says otherwise.
  */
 int fp8gemm_launch_tuned(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
                          float *out, int algo, int variant, int split_k, void *stream);
@@ -81,7 +84,7 @@ int fp8gemm_num_variants(int algo);
 /* Which family FP8GEMM_ALGO_AUTO picks for a shape (pure host logic). */
 int fp8gemm_select_algo(int m, int k, int n);
 
-/* Bytes of device scratch the split-K path of the skinny kernel keeps cached
+/* Bytes of device scratch (partial sums of K slices) the library keeps cached
  * per device for a shape (0 when the shape needs none).  The scratch is the
  * only allocation the library ever makes; it is grown on demand, reused by
  * later calls and shared by all streams of the device, so calls that overlap

@@ -12,6 +12,7 @@
 
 #include "kernel_direct.h"
 #include "kernel_ptile.h"
+#include "kernel_reduce.h"
 #include "kernel_skinny.h"
 #include "kernel_tile.h"
 
@@ -27,9 +28,10 @@ using TileP4 = TileShape<256, 256, 64, 2, 2, 4, 2>;   // persistent, 4 x 32 KiB 
 using TileP8 = TileShape<256, 256, 128, 2, 4, 2, 3>;  // persistent, 8 waves, 128x64 per wave
 using TileS2 = TileShape<128, 128, 128, 2, 2, 2, 3>;  // one tile per workgroup, for small problems
 using TileS4 = TileShape<128, 128, 128, 2, 2, 4, 3>;
-using TileH2 = TileShape<128, 256, 128, 2, 2, 2, 3>;  // persistent, half-height tile: more tiles for short-m problems
+using TileH3 = TileShape<128, 256, 128, 2, 2, 3, 3>;  // persistent, half-height tile, 3 x 48 KiB ring
 using TileQ2 = TileShape<128, 128, 128, 2, 2, 2, 3>;  // persistent, quarter tile
-constexpr int kNumTileVariants = 7;               // 0 P2, 1 P4, 2 P8, 3 S2, 4 S4, 5 H2, 6 Q2
+using TileS64 = TileShape<128, 128, 64, 2, 2, 4, 2>;  // one tile per workgroup, 64-byte K tiles
+constexpr int kNumTileVariants = 8;               // 0 P2, 1 P4, 2 P8, 3 S2, 4 S4, 5 H3, 6 Q2, 7 S64
 
 // Skinny kernel shapes: <MT, TN, BK, stages>.
 template <int MT, int TN>
@@ -89,6 +91,22 @@ hipError_t allow_lds(Kernel kernel, int bytes)
                                hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
 }
 
+// out[i] = sum over the nsplit planes of ws, on `stream`
+hipError_t launch_reduce(const float *ws, float *out, size_t count, int nsplit, hipStream_t stream)
+{
+    const bool vec = count % 4 == 0 &&
+                     ((reinterpret_cast<uintptr_t>(ws) | reinterpret_cast<uintptr_t>(out)) % 16) == 0;
+    if (vec) {
+        const size_t count4 = count / 4;
+        hipLaunchKernelGGL(gemm_splitk_reduce4_kernel, dim3((unsigned)((count4 + 255) / 256)), dim3(256), 0, stream,
+                           reinterpret_cast<const v4f *>(ws), reinterpret_cast<v4f *>(out), count4, nsplit);
+    } else {
+        hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
+                           ws, out, count, nsplit);
+    }
+    return hipGetLastError();
+}
+
 // ------------------------------------------------------------------ direct
 template <int AF, int BF>
 hipError_t launch_direct(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
@@ -125,42 +143,65 @@ hipError_t launch_tile_shape(int m, int k, int n, const uint8_t *a, const uint8_
     return hipGetLastError();
 }
 
-// persistent form: one workgroup per CU walks the tiles of its XCD
+// Super-block of tiles that the 32 CUs of one XCD work on together: 4 x 8 when the
+// grid of tiles allows, else as close to 32 tiles as it gets.
+struct TileBlocks {
+    int tiles_m, tiles_n, GM, GN, nb;
+};
+TileBlocks tile_blocks(int m, int n, int bm, int bn)
+{
+    TileBlocks t;
+    t.tiles_m = (m + bm - 1) / bm;
+    t.tiles_n = (n + bn - 1) / bn;
+    t.GM = t.tiles_m < 4 ? t.tiles_m : 4;
+    t.GN = t.tiles_n < 32 / t.GM ? t.tiles_n : 32 / t.GM;
+    t.GM = t.tiles_m < 32 / t.GN ? t.tiles_m : 32 / t.GN;
+    t.nb = ((t.tiles_m + t.GM - 1) / t.GM) * ((t.tiles_n + t.GN - 1) / t.GN);
+    return t;
+}
+
+// persistent form: one workgroup per CU walks the (tile, K slice) items of its XCD;
+// with nsplit > 1 the slices' partial sums go through the scratch buffer
 template <class S, int AF, int BF>
 hipError_t launch_ptile_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
-                              hipStream_t stream)
+                              int nsplit, int rotate, hipStream_t stream)
 {
-    if (k % S::BK != 0) return hipErrorInvalidValue;
-    const int tiles_m = (m + S::BM - 1) / S::BM;
-    const int tiles_n = (n + S::BN - 1) / S::BN;
-    // 32 tiles = the 32 CUs of one XCD; 4 x 8 when the grid of tiles allows, else as
-    // close to 32 as it gets
-    int GM = tiles_m < 4 ? tiles_m : 4;
-    int GN = tiles_n < 32 / GM ? tiles_n : 32 / GM;
-    GM = tiles_m < 32 / GN ? tiles_m : 32 / GN;
-    const int nb = ((tiles_m + GM - 1) / GM) * ((tiles_n + GN - 1) / GN);
-    const int rounds = (nb + 7) / 8;
-    const int grid = 8 * GM * GN;
+    if (k % S::BK != 0 || nsplit < 1 || nsplit > k / S::BK) return hipErrorInvalidValue;
+    const TileBlocks t = tile_blocks(m, n, S::BM, S::BN);
+    const int rounds = (t.nb * nsplit + 7) / 8;
+    const int grid = 8 * t.GM * t.GN;
+    float *dst = out;
+    if (nsplit > 1) {
+        void *ws = nullptr;
+        hipError_t e = scratch_get((size_t)nsplit * m * n * sizeof(float), &ws);
+        if (e != hipSuccess) return e;
+        dst = static_cast<float *>(ws);
+    }
     auto kernel = gemm_ptile_kernel<S, AF, BF>;
     hipError_t e = allow_lds(kernel, S::PTILE_LDS_BYTES);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(S::THREADS), S::PTILE_LDS_BYTES, stream,
-                       m, k, n, a, b, out, tiles_m, tiles_n, GM, GN, rounds);
-    return hipGetLastError();
+                       m, k, n, a, b, dst, t.tiles_m, t.tiles_n, t.GM, t.GN, rounds, nsplit, rotate);
+    e = hipGetLastError();
+    if (e != hipSuccess || nsplit == 1) return e;
+    return launch_reduce(dst, out, (size_t)m * n, nsplit, stream);
 }
 
 template <int AF, int BF>
 hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
-                       int variant, hipStream_t stream)
+                       int variant, int nsplit, int rotate, hipStream_t stream)
 {
+    const bool persistent = !(variant == 3 || variant == 4 || variant == 7);
+    if (!persistent && nsplit != 1) return hipErrorInvalidValue;   // K slices only in the persistent kernels
     switch (variant) {
-    case 0: return launch_ptile_shape<TileP2, AF, BF>(m, k, n, a, b, out, stream);
-    case 1: return launch_ptile_shape<TileP4, AF, BF>(m, k, n, a, b, out, stream);
-    case 2: return launch_ptile_shape<TileP8, AF, BF>(m, k, n, a, b, out, stream);
+    case 0: return launch_ptile_shape<TileP2, AF, BF>(m, k, n, a, b, out, nsplit, rotate, stream);
+    case 1: return launch_ptile_shape<TileP4, AF, BF>(m, k, n, a, b, out, nsplit, rotate, stream);
+    case 2: return launch_ptile_shape<TileP8, AF, BF>(m, k, n, a, b, out, nsplit, rotate, stream);
     case 3: return launch_tile_shape<TileS2, AF, BF>(m, k, n, a, b, out, stream);
     case 4: return launch_tile_shape<TileS4, AF, BF>(m, k, n, a, b, out, stream);
-    case 5: return launch_ptile_shape<TileH2, AF, BF>(m, k, n, a, b, out, stream);
-    case 6: return launch_ptile_shape<TileQ2, AF, BF>(m, k, n, a, b, out, stream);
+    case 5: return launch_ptile_shape<TileH3, AF, BF>(m, k, n, a, b, out, nsplit, rotate, stream);
+    case 6: return launch_ptile_shape<TileQ2, AF, BF>(m, k, n, a, b, out, nsplit, rotate, stream);
+    case 7: return launch_tile_shape<TileS64, AF, BF>(m, k, n, a, b, out, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -170,7 +211,7 @@ struct SkinnyPlan {
     int mt, tn, variant, nsplit;
 };
 
-template <class S, int AF, int BF, int DBG = 0>
+template <class S, int AF, int BF>
 hipError_t launch_skinny_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
                                int nsplit, hipStream_t stream)
 {
@@ -185,17 +226,14 @@ hipError_t launch_skinny_shape(int m, int k, int n, const uint8_t *a, const uint
         if (e != hipSuccess) return e;
         dst = static_cast<float *>(ws);
     }
-    auto kernel = gemm_skinny_kernel<S, AF, BF, DBG>;
+    auto kernel = gemm_skinny_kernel<S, AF, BF>;
     hipError_t e = allow_lds(kernel, S::LDS_BYTES);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3((unsigned)(ngroups * nsplit)), dim3(64), S::LDS_BYTES, stream,
                        m, k, n, a, b, dst, ngroups, kchunk);
     e = hipGetLastError();
     if (e != hipSuccess || nsplit == 1) return e;
-    const size_t count = (size_t)m * n;
-    hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
-                       dst, out, count, nsplit);
-    return hipGetLastError();
+    return launch_reduce(dst, out, (size_t)m * n, nsplit, stream);
 }
 
 template <template <int, int> class V, int AF, int BF>
@@ -223,13 +261,6 @@ hipError_t launch_skinny(int m, int k, int n, const uint8_t *a, const uint8_t *b
     case 3: return launch_skinny_mt<SkinnyV3, AF, BF>(m, k, n, a, b, out, p, stream);
     case 4: return launch_skinny_mt<SkinnyV4, AF, BF>(m, k, n, a, b, out, p, stream);
     case 5: return launch_skinny_mt<SkinnyV5, AF, BF>(m, k, n, a, b, out, p, stream);
-#ifdef FP8GEMM_TUNING
-    case 10: return launch_skinny_shape<SkinnyV0<1, 4>, AF, BF, 1>(m, k, n, a, b, out, p.nsplit, stream);
-    case 11: return launch_skinny_shape<SkinnyV0<1, 4>, AF, BF, 2>(m, k, n, a, b, out, p.nsplit, stream);
-    case 12: return launch_skinny_shape<SkinnyV0<1, 4>, AF, BF, 3>(m, k, n, a, b, out, p.nsplit, stream);
-    case 13: return launch_skinny_shape<SkinnyV1<1, 1>, AF, BF, 3>(m, k, n, a, b, out, p.nsplit, stream);
-    case 14: return launch_skinny_shape<SkinnyV5<1, 1>, AF, BF, 3>(m, k, n, a, b, out, p.nsplit, stream);
-#endif
     default: return hipErrorInvalidValue;
     }
 }
@@ -267,15 +298,72 @@ SkinnyPlan plan_skinny(int m, int k, int n)
 int select_algo(int m, int k, int n)
 {
     if (skinny_ok(m, k, n)) return FP8GEMM_ALGO_SKINNY;
-    if (k % 128 == 0) return FP8GEMM_ALGO_TILE;
+    if (k % 64 == 0) return FP8GEMM_ALGO_TILE;
     return FP8GEMM_ALGO_DIRECT;
 }
 
-int default_tile_variant(int m, int n, int stages)
+// Which tiled kernel, how many K slices, which K-walk rotation.
+struct TilePlan {
+    int variant, nsplit, rotate;
+};
+
+// Cost model behind the choice, in microseconds, fitted to MI355X timings of the
+// persistent kernels (operands cold in the caches, 128-byte K tiles):
+//   main kernel = max(rounds * (k_tiles_per_item * per_k_tile + per_item), input_bytes / stream_rate)
+//   K slices add one reduction pass over (nsplit + 1) planes of C.
+// rounds follows the kernel's own walk: 8 XCDs, each taking one super-block of tiles
+// per round.  The model only has to rank the candidates, not to predict the time.
+struct PtileCost {
+    int variant, bm, bn;
+    double per_k_tile, per_item, stream_rate;   // us, us, bytes per us
+};
+constexpr PtileCost kPtileCosts[] = {
+    {0, 256, 256, 1.33, 15.0, 3.4e6},
+    {5, 128, 256, 0.80, 8.0, 4.8e6},
+    {6, 128, 128, 0.56, 5.7, 3.0e6},
+};
+constexpr int kSplitChoices[] = {1, 2, 3, 4, 6, 8, 12, 16};
+constexpr int kMinKTilesPerSlice = 12;
+constexpr size_t kMaxSplitScratch = (size_t)1 << 30;
+
+TilePlan plan_tile(int m, int k, int n, int stages)
 {
     const long tiles256 = (long)((m + 255) / 256) * ((n + 255) / 256);
-    if (tiles256 < 192) return stages == 2 ? 3 : 4;   // small problem: 128x128 tiles fill more CUs
-    return stages == 2 ? 0 : 1;
+    const bool small = tiles256 < 192;
+    TilePlan best = {0, 1, 2};
+    if (k % 128 != 0) {                 // odd number of 64-byte K tiles
+        best.variant = small ? 7 : 1;
+        return best;
+    }
+    if (stages == 4) {                  // the 4-deep rings: one shape for big problems, one for small
+        best.variant = small ? 4 : 1;
+        return best;
+    }
+    const int kt = k / 128;
+    double best_cost = 1e30;
+    for (const PtileCost &c : kPtileCosts) {
+        const TileBlocks t = tile_blocks(m, n, c.bm, c.bn);
+        for (int split : kSplitChoices) {
+            if (split > 1 && (kt / split < kMinKTilesPerSlice ||
+                              (size_t)split * m * n * sizeof(float) > kMaxSplitScratch))
+                continue;
+            const int rounds = (t.nb * split + 7) / 8;
+            const int kt_item = (kt + split - 1) / split;
+            double cost = rounds * (kt_item * c.per_k_tile + c.per_item);
+            const double stream = ((double)m * k + (double)n * k) / c.stream_rate;
+            if (stream > cost) cost = stream;
+            if (split > 1) cost += 2.0 + (split + 1) * (double)m * n * 4.0 / 6.0e6;
+            if (cost < best_cost) {
+                best_cost = cost;
+                best.variant = c.variant;
+                best.nsplit = split;
+            }
+        }
+    }
+    // K-walk rotation: per tile column while A is small enough to stay in an XCD's L2
+    // next to the B rows in flight, else per super-block
+    best.rotate = ((size_t)m * k <= ((size_t)2 << 20)) ? 1 : 2;
+    return best;
 }
 
 template <int AF, int BF>
@@ -290,10 +378,22 @@ hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, flo
     switch (algo) {
     case FP8GEMM_ALGO_DIRECT:
         return launch_direct<AF, BF>(m, k, n, a, b, out, stream);
-    case FP8GEMM_ALGO_TILE:
-        if (!aligned || k % 128 != 0) return hipErrorInvalidValue;
-        if (variant < 0) variant = default_tile_variant(m, n, stages);
-        return launch_tile<AF, BF>(m, k, n, a, b, out, variant, stream);
+    case FP8GEMM_ALGO_TILE: {
+        if (!aligned || k % 64 != 0) return hipErrorInvalidValue;
+        TilePlan p = plan_tile(m, k, n, stages);
+        if (variant >= 0) {
+            // tuning hook: variant = shape index + 16 * (1 + K-walk rotation mode); a bare
+            // shape index keeps the plan's rotation and runs unsplit unless split_k says otherwise
+            if (variant >= 16) {
+                p.rotate = variant / 16 - 1;
+                if (p.rotate > 2) return hipErrorInvalidValue;
+            }
+            p.variant = variant % 16;
+            p.nsplit = 1;
+        }
+        if (nsplit > 0) p.nsplit = nsplit;
+        return launch_tile<AF, BF>(m, k, n, a, b, out, p.variant, p.nsplit, p.rotate, stream);
+    }
     case FP8GEMM_ALGO_SKINNY: {
         if (!aligned || !skinny_ok(m, k, n)) return hipErrorInvalidValue;
         SkinnyPlan p = plan_skinny(m, k, n);
@@ -373,9 +473,12 @@ int fp8gemm_select_algo(int m, int k, int n)
 
 size_t fp8gemm_scratch_bytes(int m, int k, int n)
 {
-    if (m <= 0 || k <= 0 || n <= 0 || select_algo(m, k, n) != FP8GEMM_ALGO_SKINNY) return 0;
-    const SkinnyPlan p = plan_skinny(m, k, n);
-    return p.nsplit > 1 ? (size_t)p.nsplit * m * n * sizeof(float) : 0;
+    if (m <= 0 || k <= 0 || n <= 0) return 0;
+    int nsplit = 1;
+    const int algo = select_algo(m, k, n);
+    if (algo == FP8GEMM_ALGO_SKINNY) nsplit = plan_skinny(m, k, n).nsplit;
+    if (algo == FP8GEMM_ALGO_TILE) nsplit = plan_tile(m, k, n, 2).nsplit;
+    return nsplit > 1 ? (size_t)nsplit * m * n * sizeof(float) : 0;
 }
 
 const char *fp8gemm_error_string(int code)

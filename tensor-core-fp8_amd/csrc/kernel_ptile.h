@@ -23,7 +23,7 @@
 // turns the epilogue into 128-bit stores.
 //
 // LDS layout, swizzle and the K-permutation freedom are as in kernel_tile.h.
-// Requirements checked by the host: K % 128 == 0, 16-byte aligned a and b.
+// Requirements checked by the host: K % BK == 0, 16-byte aligned a and b.
 #ifndef FP8GEMM_KERNEL_PTILE_H
 #define FP8GEMM_KERNEL_PTILE_H
 
@@ -68,15 +68,13 @@ __device__ __forceinline__ v4i make_buffer_resource(const void *base, unsigned l
     return r;
 }
 
-// DBG (tuning builds only, results are then wrong on purpose): bit 0 drops the
-// global loads, bit 1 the waits and barriers, bit 2 the fragment reads.
-template <class S, int AF, int BF, int DBG = 0>
+template <class S, int AF, int BF>
 __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, int N,
                                                                  const uint8_t *__restrict__ A,
                                                                  const uint8_t *__restrict__ B,
                                                                  float *__restrict__ C,
                                                                  int tiles_m, int tiles_n, int GM, int GN,
-                                                                 int rounds)
+                                                                 int rounds, int nsplit, int rotate)
 {
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, CH = S::CH, RPI = S::RPI;
     constexpr int STAGES = S::STAGES, TM = S::TM, TN = S::TN, KSTEPS = S::KSTEPS;
@@ -104,21 +102,29 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         for (int j = 0; j < 2; ++j) frag_off[s][j] = (uint32_t)(((s * 4 + 2 * fg + j) ^ sw) * 16);
     const uint32_t a_base = (uint32_t)(wm * (BM / S::WM) + fi) * BK;
     const uint32_t b_base = (uint32_t)(BM * BK) + (uint32_t)(wn * (BN / S::WN) + fi) * BK;
-    const int T = K / BK;
+    const int KT = K / BK;                         // K tiles of the whole problem
 
-    // workgroups with equal id mod 8 share an XCD (and its L2): XCD x takes the
-    // super-blocks x*rounds .. x*rounds+rounds-1, slot q of its 32 workgroups
-    // takes tile q of each super-block
+    // Work items are (super-block of tiles, K slice): with nsplit > 1 the K tiles are cut
+    // into nsplit contiguous slices and slice s writes its partial sums to the s-th M x N
+    // plane behind C (the host adds the planes up afterwards).  Workgroups with equal id
+    // mod 8 share an XCD (and its L2): XCD x takes the items x*rounds .. x*rounds+rounds-1,
+    // slot q of its 32 workgroups takes tile q of each item's super-block.
     const int xcd = blockIdx.x & 7;
     const int slot = blockIdx.x >> 3;
     const int nb_n = (tiles_n + GN - 1) / GN;
-    const int nb_total = ((tiles_m + GM - 1) / GM) * nb_n;
+    const int nb_mn = ((tiles_m + GM - 1) / GM) * nb_n;
+    const int nb_total = nb_mn * nsplit;
 
-    auto tile_of_round = [&](int r, int &tm, int &tn) -> bool {
-        const int blk = xcd * rounds + r;
-        if (r >= rounds || blk >= nb_total || slot >= GM * GN) return false;
+    // tile and K-tile range [kt0, kt0 + T) of round r; false when there is none
+    auto tile_of_round = [&](int r, int &tm, int &tn, int &slice, int &kt0, int &T) -> bool {
+        const int item = xcd * rounds + r;
+        if (r >= rounds || item >= nb_total || slot >= GM * GN) return false;
+        slice = item / nb_mn;
+        const int blk = item - slice * nb_mn;
         tm = (blk / nb_n) * GM + slot / GN;
         tn = (blk % nb_n) * GN + slot % GN;
+        kt0 = (int)((long)KT * slice / nsplit);
+        T = (int)((long)KT * (slice + 1) / nsplit) - kt0;
         return tm < tiles_m && tn < tiles_n;
     };
 
@@ -139,15 +145,30 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
     const uint32_t ldsA = lds_base + (uint32_t)(wave * S::A_LOADS * RPI * BK);
     const uint32_t ldsB = lds_base + (uint32_t)(BM * BK + wave * S::B_LOADS * RPI * BK);
     v4i rsA = {0, 0, 0, 0}, rsB = {0, 0, 0, 0};
-    auto plan_loads = [&](int tile_m, int tile_n) {
+    // K walk of the planned item: K tiles kt_base + ((t + kt_rot) mod kt_count), t = 0, 1, ..
+    // The rotation kt_rot only reorders the fp32 sum.  Workgroups that walk K in step read,
+    // at any moment, addresses that agree in the bits below the row stride; with a
+    // power-of-two K those are the bits that select the HBM channel, so the whole chip
+    // would queue on a few channels at a time.  rotate == 1 starts every tile column at
+    // its own K tile (the workgroups of a column still share their B rows through L2; A
+    // must then be small enough to stay in L2), rotate == 2 every super-block (all
+    // sharing inside an XCD is kept), 0 leaves the walk alone.
+    int kt_base = 0, kt_rot = 0, kt_count = 1;
+    auto plan_loads = [&](int tile_m, int tile_n, int kt0, int count, int item) {
         const int m0 = tile_m * BM, n0 = tile_n * BN;
         rsA = make_buffer_resource(A + (size_t)m0 * K, (unsigned long long)(M - m0) * (unsigned long long)K);
         rsB = make_buffer_resource(B + (size_t)n0 * K, (unsigned long long)(N - n0) * (unsigned long long)K);
+        kt_base = kt0;
+        kt_count = count;
+        const unsigned key = rotate == 1 ? (unsigned)tile_n : (unsigned)item;
+        // (the division runs on the vector unit; the result is the same in every lane)
+        kt_rot = rotate == 0 ? 0 : __builtin_amdgcn_readfirstlane((int)(((key * 2654435761u) >> 8) % (unsigned)count));
     };
-    // load number j (0 .. LOADS-1) of K tile `ktile` into ring slot `stage`
+    // load number j (0 .. LOADS-1) of step `ktile` of the planned item's K walk into ring slot `stage`
     auto issue_load = [&](int j, int ktile, int stage) {
-        if (DBG & 1) return;
-        const uint32_t koff = (uint32_t)(ktile * BK);
+        int kk = ktile + kt_rot;
+        kk = kk >= kt_count ? kk - kt_count : kk;
+        const uint32_t koff = (uint32_t)((kt_base + kk) * BK);
         const uint32_t sbase = (uint32_t)(stage * S::STAGE_BYTES);
         if (j < S::A_LOADS)
             buffer_load_lds_b128(rsA, ldsA + sbase + (uint32_t)(j * RPI * BK), ld_off[j], koff);
@@ -159,10 +180,10 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         for (int j = 0; j < S::LOADS; ++j) issue_load(j, ktile, stage);
     };
 
-    int tile_m = 0, tile_n = 0;
-    bool have = tile_of_round(0, tile_m, tile_n);
+    int tile_m = 0, tile_n = 0, slice = 0, kt0 = 0, T = 0;
+    bool have = tile_of_round(0, tile_m, tile_n, slice, kt0, T);
     if (have) {
-        plan_loads(tile_m, tile_n);
+        plan_loads(tile_m, tile_n, kt0, T, xcd * rounds + 0);
 #pragma unroll
         for (int t = 0; t < STAGES - 1; ++t)
             if (t < T) issue_all_loads(t, t);
@@ -171,9 +192,9 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
     for (int r = 0; r < rounds; ++r) {
         if (!have) {
             // nothing here this round; still look at the next one
-            have = tile_of_round(r + 1, tile_m, tile_n);
+            have = tile_of_round(r + 1, tile_m, tile_n, slice, kt0, T);
             if (have) {
-                plan_loads(tile_m, tile_n);
+                plan_loads(tile_m, tile_n, kt0, T, xcd * rounds + r + 1);
 #pragma unroll
                 for (int t = 0; t < STAGES - 1; ++t)
                     if (t < T) issue_all_loads(t, t);
@@ -181,6 +202,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
             continue;
         }
         const int m0 = tile_m * BM, n0 = tile_n * BN;
+        float *__restrict__ Cout = C + (size_t)slice * ((size_t)M * (size_t)N);
 
         v16f acc[TM][TN];
 #pragma unroll
@@ -192,19 +214,10 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
 
         // fragment sets: frag[p][0..TM-1] = A blocks, frag[p][TM..TM+TN-1] = B blocks
         v4i frag[2][TM + TN][2];
-        if (DBG & 4) {
-#pragma unroll
-            for (int p = 0; p < 2; ++p)
-#pragma unroll
-                for (int i = 0; i < TM + TN; ++i)
-#pragma unroll
-                    for (int h = 0; h < 2; ++h) frag[p][i][h] = v4i{tid + i, tid * 3 + h, i, p};
-        }
         // read number q (0 .. NREADS-1) of K step ks of ring slot `stage` into set p.
         // Order: B0, A0, B1 .. B(TN-1), A1 .. A(TM-1), the order the MFMAs need them.
         auto issue_read = [&](auto pc, int q, int stage, int ks) {
             constexpr int P = decltype(pc)::value;
-            if (DBG & 4) return;
             const int f = q >> 1, h = q & 1;
             int idx;           // index into frag[P]
             if (f == 0) idx = TM;
@@ -243,7 +256,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                 rstage = (t + 1) % STAGES;
                 rks = 0;
                 reads = next;
-                if (next && !(DBG & 2)) {
+                if (next) {
                     // every fragment read of K tile t has been issued; once they have
                     // returned this wave no longer needs the ring slot
                     wait_lgkmcnt0();
@@ -288,7 +301,8 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                 kstep(I1{}, I1{}, t + 1 < T, false, t);
             }
         } else {
-            // K % 128 == 0 makes the number of 64-byte K tiles even: steps go in pairs
+            // one K step per K tile: the fragment sets alternate from K tile to K tile, so
+            // K tiles go in pairs (an odd count ends on a single one)
             const int t_pair_end = t_load_end & ~1;
             int t = 0;
             for (; t < t_pair_end; t += 2) {
@@ -304,13 +318,13 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         // all waves are done reading LDS for this tile before the ring is reused
         wait_lgkmcnt0();
         __syncthreads();
-        int next_m = 0, next_n = 0;
-        have = tile_of_round(r + 1, next_m, next_n);
+        int next_m = 0, next_n = 0, next_slice = 0, next_kt0 = 0, next_T = 0;
+        have = tile_of_round(r + 1, next_m, next_n, next_slice, next_kt0, next_T);
         if (have) {
-            plan_loads(next_m, next_n);
+            plan_loads(next_m, next_n, next_kt0, next_T, xcd * rounds + r + 1);
 #pragma unroll
             for (int t = 0; t < STAGES - 1; ++t)
-                if (t < T) issue_all_loads(t, t);
+                if (t < next_T) issue_all_loads(t, t);
         }
 
         // ---- epilogue: registers -> C -------------------------------------------
@@ -318,21 +332,8 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         const int wrow0 = m0 + wm * (BM / S::WM);
         const int wcol0 = n0 + wn * (BN / S::WN);
         const bool full = (m0 + BM <= M) && (n0 + BN <= N) && (N % 4 == 0) &&
-                          (reinterpret_cast<uintptr_t>(C) % 16 == 0);
-        bool skip_store = false;
-        if (DBG & 16) {
-            // tuning: no stores; the data-dependent test keeps the computation alive
-            float chk = 0.0f;
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int q = 0; q < 16; ++q) chk += acc[i][j][q];
-            skip_store = (chk != 12345.678f);
-        }
-        if (skip_store) {
-        } else if (full) {
+                          (reinterpret_cast<uintptr_t>(Cout) % 16 == 0);
+        if (full) {
             // Each wave transposes its results through a private strip of LDS (the part of
             // the ring the next tile's first loads do not use, plus the LDS above the ring)
             // so that every store instruction writes whole contiguous row segments of C:
@@ -358,7 +359,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
 #pragma unroll
                     for (int r0 = 0; r0 < 32; r0 += RPI_ST) {
                         const v4f v = *reinterpret_cast<const v4f *>(stg + (r0 + rl) * ROWB + cl * 16);
-                        float *dst = C + (size_t)(wrow0 + i * 32 + r0 + rl) * N + wcol0 + c0 + cl * 4;
+                        float *dst = Cout + (size_t)(wrow0 + i * 32 + r0 + rl) * N + wcol0 + c0 + cl * 4;
                         *reinterpret_cast<v4f *>(dst) = v;
                     }
                 }
@@ -372,13 +373,16 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
 #pragma unroll
                         for (int q = 0; q < 16; ++q) {
                             const int col = wcol0 + j * 32 + 8 * (q >> 2) + 4 * fg + (q & 3);
-                            if (col < N) C[(size_t)row * N + col] = acc[i][j][q];
+                            if (col < N) Cout[(size_t)row * N + col] = acc[i][j][q];
                         }
                 }
             }
         }
         tile_m = next_m;
         tile_n = next_n;
+        slice = next_slice;
+        kt0 = next_kt0;
+        T = next_T;
     }
 }
 

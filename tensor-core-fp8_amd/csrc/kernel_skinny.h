@@ -12,8 +12,8 @@
 // are never stored.
 //
 // With nsplit == 1 results go straight to C; otherwise fp32 partials go to a
-// scratch buffer ws[split][m][n] and gemm_splitk_reduce_kernel adds them in
-// ascending split order (deterministic).
+// scratch buffer ws[split][m][n] and the reduction kernel (kernel_reduce.h) adds them
+// in ascending split order (deterministic).
 //
 // Requirements checked by the host: kchunk % BK == 0, n % (16*TN) == 0,
 // m <= 16*MT, 16-byte aligned a and b.
@@ -68,9 +68,7 @@ __device__ __forceinline__ int skinny_swizzle(int row)
     return ((row & 7) ^ ((row >> 3) & 1));
 }
 
-// DBG (tuning builds only, wrong results on purpose): bit 0 drops the loads of A,
-// bit 1 the fragment reads and MFMAs.
-template <class S, int AF, int BF, int DBG = 0>
+template <class S, int AF, int BF>
 __global__ __launch_bounds__(64) void gemm_skinny_kernel(int M, int K, int N,
                                                          const uint8_t *__restrict__ A,
                                                          const uint8_t *__restrict__ B,
@@ -111,7 +109,7 @@ __global__ __launch_bounds__(64) void gemm_skinny_kernel(int M, int K, int N,
         int t = tt + t0;
         t = t >= T ? t - T : t;
 #pragma unroll
-        for (int j = (DBG & 1) ? S::A_LOADS : 0; j < S::LOADS; ++j)
+        for (int j = 0; j < S::LOADS; ++j)
             __builtin_amdgcn_global_load_lds((const GLOBAL_AS void *)(src[j] + (size_t)t * BK),
                                              (LDS_AS void *)(lds + stage * S::STAGE_BYTES + j * RPI * BK),
                                              16, 0, 0);
@@ -142,13 +140,13 @@ __global__ __launch_bounds__(64) void gemm_skinny_kernel(int M, int K, int N,
         // refill the stage consumed one step ago, then wait for stage t
         if (t + STAGES - 1 < T) {
             issue_loads(t + STAGES - 1, (t + STAGES - 1) % STAGES);
-            wait_vmcnt<((DBG & 1) ? S::LOADS - S::A_LOADS : S::LOADS) * (STAGES - 1)>();
+            wait_vmcnt<S::LOADS *(STAGES - 1)>();
         } else {
             wait_vmcnt<0>();
         }
         const uint8_t *st = lds + (t % STAGES) * S::STAGE_BYTES;
 #pragma unroll
-        for (int s = 0; s < ((DBG & 2) ? 0 : S::KSTEPS); ++s) {
+        for (int s = 0; s < S::KSTEPS; ++s) {
             v8i af[MT], bf[TN];
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
@@ -182,18 +180,6 @@ __global__ __launch_bounds__(64) void gemm_skinny_kernel(int M, int K, int N,
                 const int row = i * 16 + 4 * fq + r;
                 if (row < M) dst[(size_t)row * N + n0 + j * 16 + fi] = acc[i][j][r];
             }
-}
-
-// C[i] = ws[0][i] + ws[1][i] + ... in ascending split order.
-__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float *__restrict__ ws,
-                                                                 float *__restrict__ C,
-                                                                 size_t count, int nsplit)
-{
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= count) return;
-    float s = ws[i];
-    for (int p = 1; p < nsplit; ++p) s += ws[(size_t)p * count + i];
-    C[i] = s;
 }
 
 #endif  // FP8GEMM_KERNEL_SKINNY_H

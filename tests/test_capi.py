@@ -53,13 +53,17 @@ def test_kernel_selection_is_pure_host_logic(pkg):
     assert L.fp8gemm_select_algo(1, 28672, 8192) == pkg.ALGO_SKINNY
     assert L.fp8gemm_select_algo(64, 8192, 10240) == pkg.ALGO_SKINNY
     assert L.fp8gemm_select_algo(256, 8192, 28672) == pkg.ALGO_TILE
-    assert L.fp8gemm_select_algo(100, 100, 100) == pkg.ALGO_DIRECT       # k not a multiple of 128
+    assert L.fp8gemm_select_algo(100, 100, 100) == pkg.ALGO_DIRECT       # k not a multiple of 64
+    assert L.fp8gemm_select_algo(512, 192, 512) == pkg.ALGO_TILE         # odd count of 64-byte K tiles
     assert L.fp8gemm_select_algo(16, 100, 64) == pkg.ALGO_DIRECT
     assert L.fp8gemm_select_algo(0, 1, 1) == -1
     assert L.fp8gemm_num_variants(pkg.ALGO_TILE) >= 2 and L.fp8gemm_num_variants(pkg.ALGO_SKINNY) >= 1
     assert L.fp8gemm_scratch_bytes(8192, 8192, 8192) == 0
     s = L.fp8gemm_scratch_bytes(16, 28672, 8192)
     assert s % (16 * 8192 * 4) == 0        # whole partial-sum planes, or none
+    # few tiles and a long K: the tiled kernels cut K into slices, whole planes of partial sums
+    s = L.fp8gemm_scratch_bytes(256, 28672, 8192)
+    assert s >= 2 * 256 * 8192 * 4 and s % (256 * 8192 * 4) == 0
 
 
 def test_generators_are_reproducible_and_counter_based(pkg):

@@ -107,7 +107,7 @@ def test_normal_inputs_within_fp32_reordering_bound(pkg, oracle, fa, fb, algo, s
     assert worst < 0.25
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("shape", [(256, 256, 256), (300, 512, 200), (1000, 1024, 900), (513, 384, 257), (64, 128, 2048)])
 def test_every_tile_variant(pkg, oracle, variant, shape):
     """Each compiled shape of the tiled kernels (persistent and one-tile-per-workgroup),
@@ -119,6 +119,40 @@ def test_every_tile_variant(pkg, oracle, variant, shape):
     B = np.where(((B >> 2) & 0x1F) > 24, B & 0x83 | 0x3C, B).astype(np.uint8)
     C = run_gpu(pkg, A, 0, B, 1, algo=ALGOS["tile"], variant=variant)
     assert_within_bound(oracle, C, A, 0, B, 1, hw_term=True)
+
+
+@pytest.mark.parametrize("variant,split", [(0, 2), (0, 3), (1, 5), (5, 4), (5, 7), (6, 2), (6, 16), (2, 2)])
+@pytest.mark.parametrize("shape", [(256, 2048, 512), (300, 4096, 200), (1000, 2304, 900), (128, 8192, 2048)])
+def test_tile_k_slices(pkg, oracle, variant, split, shape):
+    """Persistent tiled kernels with the K range cut into slices whose partial sums are
+    added by the reduction kernel (uneven slices included), on shapes that overhang the tile."""
+    M, K, N = shape
+    A = pkg.fill((M, K), 1, seed=0xA11CE + K + split, dist="normal", sigma=4.0)
+    B = pkg.fill((N, K), 0, seed=0xB0B + K + split, dist="normal", sigma=4.0)
+    C = run_gpu(pkg, A, 1, B, 0, algo=ALGOS["tile"], variant=variant, split_k=split)
+    worst = assert_within_bound(oracle, C, A, 1, B, 0)
+    assert worst < 0.25
+
+
+@pytest.mark.parametrize("variant", [1, 7, None])
+@pytest.mark.parametrize("shape", [(256, 64, 256), (300, 192, 200), (1100, 448, 2100), (2048, 8256, 2304)])
+def test_odd_count_of_64_byte_k_tiles(pkg, oracle, variant, shape):
+    """k % 64 == 0 but k % 128 != 0 (the reference's own requirement is k % 64 == 0,
+    GEMM/src/gemm.cu:45-47): the tiled kernels with 64-byte K tiles take it, whether picked
+    by hand or by the automatic selection."""
+    M, K, N = shape
+    assert pkg.lib().fp8gemm_select_algo(M, K, N) == ALGOS["tile"]
+    A = pkg.fill((M, K), 0, seed=0xA11CE + K, dist="normal", sigma=4.0)
+    B = pkg.fill((N, K), 1, seed=0xB0B + K, dist="normal", sigma=4.0)
+    if variant is None:
+        C = run_gpu(pkg, A, 0, B, 1)
+    else:
+        C = run_gpu(pkg, A, 0, B, 1, algo=ALGOS["tile"], variant=variant)
+    rows = None if M * N * K < 2 ** 31 else np.arange(0, M, 16, dtype=np.int32)
+    # one or a few MFMAs per output: their internal alignment window shows next to the
+    # K-proportional bound
+    worst = assert_within_bound(oracle, C, A, 0, B, 1, rows=rows, hw_term=K < 1024)
+    assert worst < 0.25
 
 
 @pytest.mark.parametrize("stages", [2, 4])
