@@ -40,7 +40,7 @@ class Fp8GemmError(RuntimeError):
 
 def build(jobs=8):
     """Compile the library and the harness for gfx950 (hipcc; no GPU needed)."""
-    subprocess.check_call(["make", "-C", HARNESS_DIR, "-j", str(jobs), "lib", "gemm"])
+    subprocess.check_call(["make", "-C", HARNESS_DIR, "-j", str(jobs), "lib", "gemm", "hipblaslt"])
 
 
 def lib():

@@ -136,3 +136,26 @@ def test_accumulation_stress_mixed_pairings(pkg, oracle, fa, fb):
     worst = check_rows(oracle, out, A, fa, B, fb, residue_rows(M))
     assert worst < 0.1
     check_sums(oracle, out, dA, fa, dB, fb)
+
+
+def test_a_operand_beyond_2_31_elements(pkg, oracle):
+    """A with more than 2^31 elements (65600 x 32768): the rows past the 2 GiB offset are
+    checked against the oracle, the rest through sampled rows."""
+    M, K, N = 65600, 32768, 512
+    A = pkg.fill((M, K), 0, seed=0xA11CE + 6, dist="normal")
+    B = pkg.fill((N, K), 0, seed=0xB0B + 6, dist="normal")
+    out, dA, dB = gpu_gemm(pkg, A, 0, B, 0)
+    rows = np.concatenate([np.arange(0, 65536, 1021), np.arange(65536, M)]).astype(np.int32)
+    worst = check_rows(oracle, out, A, 0, B, 0, rows)
+    assert worst < 0.05
+
+
+def test_c_beyond_2_31_elements(pkg, oracle):
+    """C with more than 2^31 elements (65536 x 32832 fp32, 8.6 GB): sampled rows, the last
+    ones included, element by element."""
+    M, K, N = 65536, 512, 32832
+    A = pkg.fill((M, K), 1, seed=0xA11CE + 7, dist="normal")
+    B = pkg.fill((N, K), 0, seed=0xB0B + 7, dist="normal")
+    out, dA, dB = gpu_gemm(pkg, A, 1, B, 0)
+    rows = np.concatenate([np.arange(0, M, 997), np.arange(M - 40, M)]).astype(np.int32)
+    check_rows(oracle, out, A, 1, B, 0, rows)      # the bound itself; K is short, so no margin is asked for
