@@ -25,7 +25,7 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E peak, GB/s
 # HBM bytes moved by one 8192^3 launch of the tiled kernel, from rocprofv3
 # FETCH_SIZE / WRITE_SIZE counter runs scaled by the reading of a plain copy
 # kernel of known size (summary under profiles/).
-TRAFFIC_BYTES_8192 = (2 * 394178 + 308809) * 1024   # FETCH_SIZE x 2.0 (copy-kernel scale) + WRITE_SIZE x 1.0, KiB -> bytes
+TRAFFIC_BYTES_8192 = (2 * 392249 + 262144) * 1024   # FETCH_SIZE x 2.0 (copy-kernel scale) + WRITE_SIZE x 1.0, KiB -> bytes
 
 
 def load_package():
@@ -65,8 +65,8 @@ def time_launches(torch, fn, steps, warmup):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=300)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host CPU leg")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel that FETCH_SIZE / WRITE_SIZE "
