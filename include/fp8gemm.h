@@ -84,6 +84,13 @@ int fp8gemm_num_variants(int algo);
 /* Which family FP8GEMM_ALGO_AUTO picks for a shape (pure host logic). */
 int fp8gemm_select_algo(int m, int k, int n);
 
+/* What fp8gemm_launch would run for a shape with 16-byte aligned operands (pure
+ * host logic): plan[0] = family (FP8GEMM_ALGO_*), plan[1] = compiled shape variant
+ * of that family, plan[2] = number of K slices (1 = none, no scratch), plan[3] =
+ * columns of C per wave (skinny family) or K-walk rotation mode (tiled family).
+ * Returns 0, or hipErrorInvalidValue for bad arguments. */
+int fp8gemm_plan(int m, int k, int n, int stages, int plan[4]);
+
 /* Bytes of device scratch (partial sums of K slices) the library keeps cached
  * per device for a shape (0 when the shape needs none).  The scratch is the
  * only allocation the library ever makes; it is grown on demand, reused by

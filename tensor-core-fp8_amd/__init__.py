@@ -74,6 +74,8 @@ def lib():
     L.fp8gemm_num_variants.argtypes = [ci]
     L.fp8gemm_select_algo.restype = ci
     L.fp8gemm_select_algo.argtypes = [ci, ci, ci]
+    L.fp8gemm_plan.restype = ci
+    L.fp8gemm_plan.argtypes = [ci, ci, ci, ci, ctypes.POINTER(ci)]
     L.fp8gemm_scratch_bytes.restype = ctypes.c_size_t
     L.fp8gemm_scratch_bytes.argtypes = [ci, ci, ci]
     L.fp8gemm_error_string.restype = ctypes.c_char_p
@@ -102,6 +104,14 @@ def lib():
 def check(code):
     if code != 0:
         raise Fp8GemmError("fp8gemm error %d: %s" % (code, lib().fp8gemm_error_string(code).decode()))
+
+
+def plan(m, k, n, stages=2):
+    """(family, variant, K slices, columns per wave | rotation mode) that the automatic
+    selection uses for a shape."""
+    out = (ctypes.c_int * 4)()
+    check(lib().fp8gemm_plan(m, k, n, stages, out))
+    return tuple(out)
 
 
 # ---------------------------------------------------------------- host codec

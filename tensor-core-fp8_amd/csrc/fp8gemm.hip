@@ -31,7 +31,8 @@ using TileS4 = TileShape<128, 128, 128, 2, 2, 4, 3>;
 using TileH3 = TileShape<128, 256, 128, 2, 2, 3, 3>;  // persistent, half-height tile, 3 x 48 KiB ring
 using TileQ2 = TileShape<128, 128, 128, 2, 2, 2, 3>;  // persistent, quarter tile
 using TileS64 = TileShape<128, 128, 64, 2, 2, 4, 2>;  // one tile per workgroup, 64-byte K tiles
-constexpr int kNumTileVariants = 8;               // 0 P2, 1 P4, 2 P8, 3 S2, 4 S4, 5 H3, 6 Q2, 7 S64
+using TileW3 = TileShape<256, 128, 128, 2, 2, 3, 3>;  // persistent, half-width tile, 3 x 48 KiB ring
+constexpr int kNumTileVariants = 9;               // 0 P2, 1 P4, 2 P8, 3 S2, 4 S4, 5 H3, 6 Q2, 7 S64, 8 W3
 
 // Skinny kernel shapes: <MT, TN, BK, stages>.
 template <int MT, int TN>
@@ -143,20 +144,40 @@ hipError_t launch_tile_shape(int m, int k, int n, const uint8_t *a, const uint8_
     return hipGetLastError();
 }
 
-// Super-block of tiles that the 32 CUs of one XCD work on together: 4 x 8 when the
-// grid of tiles allows, else as close to 32 tiles as it gets.
+// Super-block of GM x GN tiles that the CUs of one XCD work on together (at most 32
+// tiles, one per CU).  Chosen for: fewest rounds of the persistent walk; then the
+// smallest block, so that a problem with few tiles spreads over all eight XCDs (their
+// L2s and fabric links) instead of filling some and leaving others idle; then the
+// fewest operand panels per tile (1/GM + 1/GN), i.e. the most sharing inside the L2.
 struct TileBlocks {
-    int tiles_m, tiles_n, GM, GN, nb;
+    int tiles_m, tiles_n, GM, GN, nb, rounds;
 };
-TileBlocks tile_blocks(int m, int n, int bm, int bn)
+TileBlocks tile_blocks(int m, int n, int bm, int bn, int nsplit)
 {
     TileBlocks t;
     t.tiles_m = (m + bm - 1) / bm;
     t.tiles_n = (n + bn - 1) / bn;
-    t.GM = t.tiles_m < 4 ? t.tiles_m : 4;
-    t.GN = t.tiles_n < 32 / t.GM ? t.tiles_n : 32 / t.GM;
-    t.GM = t.tiles_m < 32 / t.GN ? t.tiles_m : 32 / t.GN;
-    t.nb = ((t.tiles_m + t.GM - 1) / t.GM) * ((t.tiles_n + t.GN - 1) / t.GN);
+    t.GM = t.GN = 1;
+    t.nb = t.tiles_m * t.tiles_n;
+    t.rounds = 0;
+    double best_share = 0.0;
+    for (int gm = 1; gm <= 8 && gm <= t.tiles_m; ++gm)
+        for (int gn = 1; gn <= 32 / gm && gn <= t.tiles_n; ++gn) {
+            const long nb = (long)((t.tiles_m + gm - 1) / gm) * ((t.tiles_n + gn - 1) / gn);
+            const long rounds = (nb * nsplit + 7) / 8;
+            if (rounds > 0x7fffffff) continue;
+            const double share = 1.0 / gm + 1.0 / gn;
+            const bool better = t.rounds == 0 || rounds < t.rounds ||
+                                (rounds == t.rounds && (gm * gn < t.GM * t.GN ||
+                                                        (gm * gn == t.GM * t.GN && share < best_share)));
+            if (better) {
+                t.GM = gm;
+                t.GN = gn;
+                t.nb = (int)nb;
+                t.rounds = (int)rounds;
+                best_share = share;
+            }
+        }
     return t;
 }
 
@@ -167,8 +188,8 @@ hipError_t launch_ptile_shape(int m, int k, int n, const uint8_t *a, const uint8
                               int nsplit, int rotate, hipStream_t stream)
 {
     if (k % S::BK != 0 || nsplit < 1 || nsplit > k / S::BK) return hipErrorInvalidValue;
-    const TileBlocks t = tile_blocks(m, n, S::BM, S::BN);
-    const int rounds = (t.nb * nsplit + 7) / 8;
+    const TileBlocks t = tile_blocks(m, n, S::BM, S::BN, nsplit);
+    const int rounds = t.rounds;
     const int grid = 8 * t.GM * t.GN;
     float *dst = out;
     if (nsplit > 1) {
@@ -202,6 +223,7 @@ hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, 
     case 5: return launch_ptile_shape<TileH3, AF, BF>(m, k, n, a, b, out, nsplit, rotate, stream);
     case 6: return launch_ptile_shape<TileQ2, AF, BF>(m, k, n, a, b, out, nsplit, rotate, stream);
     case 7: return launch_tile_shape<TileS64, AF, BF>(m, k, n, a, b, out, stream);
+    case 8: return launch_ptile_shape<TileW3, AF, BF>(m, k, n, a, b, out, nsplit, rotate, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -271,23 +293,30 @@ bool skinny_ok(int m, int k, int n)
 }
 
 // Picks columns per wave, LDS shape and split-K factor.  Measured on MI355X with
-// operands that are cold in every cache: the HBM pipe is fullest with one to two
-// fat streams per CU (256..512 streams, each with a deep LDS ring) rather than many
-// thin ones; a split-K pass costs 10 % and more, so it is used only when the
-// columns alone give too few streams; long K steps (512 bytes per row and load
-// group) help a little.
+// operands that are cold in every cache.  Up to 32 rows of A the HBM pipe is fullest
+// with one to two fat streams per CU (256..512 streams, each with a deep LDS ring)
+// rather than many thin ones, and a split-K pass costs 10 % and more, so K is cut only
+// when the columns alone give too few streams.  From 33 rows on a stream spends most
+// of its LDS ring on A: the widest column group (64 columns) keeps the share of B up,
+// and about two streams per CU hide the longer MFMA phases, even at the price of K
+// slices.  Long K steps (512 bytes per row and load group) help a little.
 SkinnyPlan plan_skinny(int m, int k, int n)
 {
     SkinnyPlan p;
     p.mt = (m + 15) / 16;
-    const int tn_min = (p.mt >= 3) ? 2 : 1;       // keep the re-read of A below the read of B
-    int tn = 4;
-    while (tn > 1 && (n % (16 * tn) != 0 || (n / (16 * tn) < 256 && tn > tn_min))) tn /= 2;
-    while (n % (16 * tn) != 0) tn /= 2;           // n % 16 == 0 is guaranteed by the caller
     const int ksteps = k / 128;
-    int split = 1;
-    while ((long)(n / (16 * tn)) * split < 192 && split < 16 && ksteps % (2 * split) == 0 && ksteps / (2 * split) >= 8)
-        split *= 2;
+    int tn = 4, split = 1;
+    if (p.mt >= 3) {
+        while (n % (16 * tn) != 0) tn /= 2;       // n % 16 == 0 is guaranteed by the caller
+        // slices shorter than 4 KiB of K lose more to their ramp than the extra streams gain
+        while ((long)(n / (16 * tn)) * split < 448 && split < 16 && ksteps % (2 * split) == 0 && ksteps / (2 * split) >= 32)
+            split *= 2;
+    } else {
+        while (tn > 1 && (n % (16 * tn) != 0 || n / (16 * tn) < 256)) tn /= 2;
+        while (n % (16 * tn) != 0) tn /= 2;
+        while ((long)(n / (16 * tn)) * split < 192 && split < 16 && ksteps % (2 * split) == 0 && ksteps / (2 * split) >= 8)
+            split *= 2;
+    }
     p.tn = tn;
     p.nsplit = split;
     const int kchunk = k / split;
@@ -308,8 +337,12 @@ struct TilePlan {
 };
 
 // Cost model behind the choice, in microseconds, fitted to MI355X timings of the
-// persistent kernels (operands cold in the caches, 128-byte K tiles):
-//   main kernel = max(rounds * (k_tiles_per_item * per_k_tile + per_item), input_bytes / stream_rate)
+// persistent kernels (operands cold in the caches, 128-byte K tiles; 30 shapes x 4 tile
+// shapes x 8 slice counts, the pick is within 1 % of the best measured candidate on
+// average):
+//   main kernel = max(rounds * (k_tiles_per_item * per_k_tile * load + per_item), input_bytes / stream_rate)
+//   load        = 0.6 + 0.4 * (share of the 256 CUs that have an item in a round): a chip
+//                 that is partly idle clocks higher and contends less for L2 and fabric
 //   K slices add one reduction pass over (nsplit + 1) planes of C.
 // rounds follows the kernel's own walk: 8 XCDs, each taking one super-block of tiles
 // per round.  The model only has to rank the candidates, not to predict the time.
@@ -318,9 +351,10 @@ struct PtileCost {
     double per_k_tile, per_item, stream_rate;   // us, us, bytes per us
 };
 constexpr PtileCost kPtileCosts[] = {
-    {0, 256, 256, 1.33, 15.0, 3.4e6},
-    {5, 128, 256, 0.80, 8.0, 4.8e6},
-    {6, 128, 128, 0.56, 5.7, 3.0e6},
+    {0, 256, 256, 1.45, 11.0, 3.4e6},
+    {5, 128, 256, 0.95, 8.0, 5.0e6},
+    {6, 128, 128, 0.75, 2.5, 3.2e6},
+    {8, 256, 128, 0.90, 8.0, 4.0e6},
 };
 constexpr int kSplitChoices[] = {1, 2, 3, 4, 6, 8, 12, 16};
 constexpr int kMinKTilesPerSlice = 12;
@@ -342,17 +376,22 @@ TilePlan plan_tile(int m, int k, int n, int stages)
     const int kt = k / 128;
     double best_cost = 1e30;
     for (const PtileCost &c : kPtileCosts) {
-        const TileBlocks t = tile_blocks(m, n, c.bm, c.bn);
+        // the 256 x 128 tile pays off where it holds all rows of A at once (no second
+        // row of tiles re-reading the same B rows) and is at least half full
+        if (c.variant == 8 && (m <= 128 || m > 256)) continue;
         for (int split : kSplitChoices) {
             if (split > 1 && (kt / split < kMinKTilesPerSlice ||
                               (size_t)split * m * n * sizeof(float) > kMaxSplitScratch))
                 continue;
-            const int rounds = (t.nb * split + 7) / 8;
+            const TileBlocks t = tile_blocks(m, n, c.bm, c.bn, split);
+            const int rounds = t.rounds;
             const int kt_item = (kt + split - 1) / split;
-            double cost = rounds * (kt_item * c.per_k_tile + c.per_item);
+            double busy = (double)t.tiles_m * t.tiles_n * split / (256.0 * rounds);
+            if (busy > 1.0) busy = 1.0;
+            double cost = rounds * (kt_item * c.per_k_tile * (0.6 + 0.4 * busy) + c.per_item);
             const double stream = ((double)m * k + (double)n * k) / c.stream_rate;
             if (stream > cost) cost = stream;
-            if (split > 1) cost += 2.0 + (split + 1) * (double)m * n * 4.0 / 6.0e6;
+            if (split > 1) cost += 4.0 + (split + 1) * (double)m * n * 4.0 / 6.0e6;
             if (cost < best_cost) {
                 best_cost = cost;
                 best.variant = c.variant;
@@ -469,6 +508,28 @@ int fp8gemm_select_algo(int m, int k, int n)
 {
     if (m <= 0 || k <= 0 || n <= 0) return -1;
     return select_algo(m, k, n);
+}
+
+int fp8gemm_plan(int m, int k, int n, int stages, int plan[4])
+{
+    if (m <= 0 || k <= 0 || n <= 0 || !plan || (stages != 2 && stages != 4)) return (int)hipErrorInvalidValue;
+    const int algo = select_algo(m, k, n);
+    plan[0] = algo;
+    plan[1] = 0;
+    plan[2] = 1;
+    plan[3] = 0;
+    if (algo == FP8GEMM_ALGO_SKINNY) {
+        const SkinnyPlan p = plan_skinny(m, k, n);
+        plan[1] = p.variant;
+        plan[2] = p.nsplit;
+        plan[3] = 16 * p.tn;
+    } else if (algo == FP8GEMM_ALGO_TILE) {
+        const TilePlan p = plan_tile(m, k, n, stages);
+        plan[1] = p.variant;
+        plan[2] = p.nsplit;
+        plan[3] = p.rotate;
+    }
+    return 0;
 }
 
 size_t fp8gemm_scratch_bytes(int m, int k, int n)

@@ -61,6 +61,20 @@ def test_kernel_selection_is_pure_host_logic(pkg):
     assert L.fp8gemm_scratch_bytes(8192, 8192, 8192) == 0
     s = L.fp8gemm_scratch_bytes(16, 28672, 8192)
     assert s % (16 * 8192 * 4) == 0        # whole partial-sum planes, or none
+    # the plan behind the automatic selection: family, variant, K slices, columns | rotation
+    assert pkg.plan(8192, 8192, 8192) == (pkg.ALGO_TILE, 0, 1, 2)          # 256x256 persistent tiles, no slices
+    assert pkg.plan(8192, 8192, 8192, stages=4)[:3] == (pkg.ALGO_TILE, 1, 1)
+    fam, var, slices, cols = pkg.plan(16, 8192, 28672)
+    assert (fam, slices, cols) == (pkg.ALGO_SKINNY, 1, 64)
+    fam, var, slices, _ = pkg.plan(256, 28672, 8192)
+    assert fam == pkg.ALGO_TILE and slices > 1
+    assert pkg.plan(100, 100, 100)[0] == pkg.ALGO_DIRECT
+    for shape in [(256, 28672, 8192), (64, 28672, 8192), (300, 4096, 500), (8192, 8192, 8192)]:
+        slices = pkg.plan(*shape)[2]
+        want = slices * shape[0] * shape[2] * 4 if slices > 1 else 0
+        assert L.fp8gemm_scratch_bytes(*shape) == want
+    out = (ctypes.c_int * 4)()
+    assert L.fp8gemm_plan(0, 1, 1, 2, out) == 1 and L.fp8gemm_plan(1, 1, 1, 3, out) == 1
     # few tiles and a long K: the tiled kernels cut K into slices, whole planes of partial sums
     s = L.fp8gemm_scratch_bytes(256, 28672, 8192)
     assert s >= 2 * 256 * 8192 * 4 and s % (256 * 8192 * 4) == 0

@@ -107,7 +107,7 @@ def test_normal_inputs_within_fp32_reordering_bound(pkg, oracle, fa, fb, algo, s
     assert worst < 0.25
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("shape", [(256, 256, 256), (300, 512, 200), (1000, 1024, 900), (513, 384, 257), (64, 128, 2048)])
 def test_every_tile_variant(pkg, oracle, variant, shape):
     """Each compiled shape of the tiled kernels (persistent and one-tile-per-workgroup),
@@ -121,7 +121,7 @@ def test_every_tile_variant(pkg, oracle, variant, shape):
     assert_within_bound(oracle, C, A, 0, B, 1, hw_term=True)
 
 
-@pytest.mark.parametrize("variant,split", [(0, 2), (0, 3), (1, 5), (5, 4), (5, 7), (6, 2), (6, 16), (2, 2)])
+@pytest.mark.parametrize("variant,split", [(0, 2), (0, 3), (1, 5), (5, 4), (5, 7), (6, 2), (6, 16), (2, 2), (8, 3)])
 @pytest.mark.parametrize("shape", [(256, 2048, 512), (300, 4096, 200), (1000, 2304, 900), (128, 8192, 2048)])
 def test_tile_k_slices(pkg, oracle, variant, split, shape):
     """Persistent tiled kernels with the K range cut into slices whose partial sums are
