@@ -73,9 +73,11 @@ int fp8gemm_launch_algo(int m, int k, int n, const void *a, int a_fmt, const voi
  * -1 = the default for the shape).  For FP8GEMM_ALGO_SKINNY, variant may add
  * 16 * columns-per-wave/16 to override the planned column count per wave; for
  * FP8GEMM_ALGO_TILE it may add 16 * (1 + r) to force the K-walk rotation mode
- * r (0 none, 1 per tile column, 2 per block of tiles).  split_k > 0 overrides
+ * r (0 none, 1 per tile column, 2 per XCD and round).  split_k > 0 overrides
  * the planned number of K slices (skinny kernel and persistent tiled kernels);
- * a forced tile variant runs unsplit unless split_k says otherwise.
+ * split_k < 0 (tiled kernels only) cuts only the tiles that do not fill a
+ * round of 256 into -split_k slices; a forced tile variant runs unsplit unless
+ * split_k says otherwise.
  */
 int fp8gemm_launch_tuned(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
                          float *out, int algo, int variant, int split_k, void *stream);
@@ -87,7 +89,8 @@ int fp8gemm_select_algo(int m, int k, int n);
 /* What fp8gemm_launch would run for a shape with 16-byte aligned operands (pure
  * host logic): plan[0] = family (FP8GEMM_ALGO_*), plan[1] = compiled shape variant
  * of that family, plan[2] = number of K slices (1 = none, no scratch), plan[3] =
- * columns of C per wave (skinny family) or K-walk rotation mode (tiled family).
+ * columns of C per wave (skinny family) or, for the tiled family, the K-walk
+ * rotation mode, plus 16 when only the tiles that do not fill a round are cut.
  * Returns 0, or hipErrorInvalidValue for bad arguments. */
 int fp8gemm_plan(int m, int k, int n, int stages, int plan[4]);
 

@@ -7,7 +7,8 @@
 // lda = k, op(B) = N with ldb = k, i.e. A row-major m x k and B stored n x k, the
 // operand layout of gemm::GEMM), per-tensor scale pointers for A and B (fp32 C and D
 // take none here), a 32 MiB workspace, the first heuristic result, `repeat` launches timed one by
-// one with events and averaged (cublas.cu:66-94), and a sweep over
+// one with events and averaged (cublas.cu:66-94; here after a warm-up and in blocks that
+// alternate between the two libraries, so that both see the same clocks), and a sweep over
 // 256, 512, .. 16384 (cublas.cu:123-130).
 //
 // Differences, on purpose:
@@ -94,13 +95,15 @@ struct Problem {
     Problem &operator=(const Problem &) = delete;
 };
 
-float average_ms(int repeat, const std::function<void()> &launch)
+// Sum of the per-launch times of `count` launches, each bracketed by its own event pair
+// and a synchronisation (the sample's way of timing, cublas.cu:66-94).
+float timed_launches_ms(int count, const std::function<void()> &launch)
 {
     hipEvent_t start, stop;
     check_hip(hipEventCreate(&start), "event");
     check_hip(hipEventCreate(&stop), "event");
     float total = 0.0f;
-    for (int i = 0; i < repeat; ++i) {
+    for (int i = 0; i < count; ++i) {
         check_hip(hipEventRecord(start, nullptr), "record");
         launch();
         check_hip(hipEventRecord(stop, nullptr), "record");
@@ -111,7 +114,29 @@ float average_ms(int repeat, const std::function<void()> &launch)
     }
     (void)hipEventDestroy(start);
     (void)hipEventDestroy(stop);
-    return total / (float)repeat;
+    return total;
+}
+
+// Times two launchers under the same conditions: the chip's clocks depend on what ran in
+// the last few milliseconds, so both are warmed up first and then timed in alternating
+// blocks instead of one after the other.
+void average_ms_pair(int repeat, const std::function<void()> &first, const std::function<void()> &second,
+                     float &ms_first, float &ms_second)
+{
+    const int warm = repeat < 10 ? repeat : 10;
+    (void)timed_launches_ms(warm, first);
+    (void)timed_launches_ms(warm, second);
+    const int blocks = repeat >= 8 ? 4 : 1;
+    float total_first = 0.0f, total_second = 0.0f;
+    int done = 0;
+    for (int blk = 0; blk < blocks; ++blk) {
+        const int count = (blk == blocks - 1) ? repeat - done : repeat / blocks;
+        total_first += timed_launches_ms(count, first);
+        total_second += timed_launches_ms(count, second);
+        done += count;
+    }
+    ms_first = total_first / (float)repeat;
+    ms_second = total_second / (float)repeat;
 }
 
 // Returns false when the library offers no algorithm for the problem.
@@ -158,8 +183,8 @@ bool run_size(hipblasLtHandle_t handle, Problem &p, int repeat, bool comparable)
         vendor();
         own();
         check_hip(hipDeviceSynchronize(), "sync");
-        const float ms_vendor = average_ms(repeat, vendor);
-        const float ms_own = average_ms(repeat, own);
+        float ms_vendor = 0.0f, ms_own = 0.0f;
+        average_ms_pair(repeat, vendor, own, ms_vendor, ms_own);
         const double flop = 2.0 * p.m * (double)p.n * p.k;
         printf("Average hipblasLtMatmul execution time %f (ms)\n", ms_vendor);
         printf("GEMM-hipblaslt-fp8: M[%d] x N[%d] x K[%d], performance = %lfGFLOPS.\n", p.m, p.n, p.k,

@@ -8,6 +8,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "kernel_direct.h"
@@ -32,7 +33,8 @@ using TileH3 = TileShape<128, 256, 128, 2, 2, 3, 3>;  // persistent, half-height
 using TileQ2 = TileShape<128, 128, 128, 2, 2, 2, 3>;  // persistent, quarter tile
 using TileS64 = TileShape<128, 128, 64, 2, 2, 4, 2>;  // one tile per workgroup, 64-byte K tiles
 using TileW3 = TileShape<256, 128, 128, 2, 2, 3, 3>;  // persistent, half-width tile, 3 x 48 KiB ring
-constexpr int kNumTileVariants = 9;               // 0 P2, 1 P4, 2 P8, 3 S2, 4 S4, 5 H3, 6 Q2, 7 S64, 8 W3
+using TileT2 = TileShape<192, 256, 128, 2, 2, 2, 3>;  // persistent, three-quarter-height tile: other tile counts
+constexpr int kNumTileVariants = 10;              // 0 P2, 1 P4, 2 P8, 3 S2, 4 S4, 5 H3, 6 Q2, 7 S64, 8 W3, 9 T2
 
 // Skinny kernel shapes: <MT, TN, BK, stages>.
 template <int MT, int TN>
@@ -84,13 +86,31 @@ hipError_t scratch_get(size_t bytes, void **out)
     return hipSuccess;
 }
 
-template <class Kernel>
+// Raises a kernel's dynamic LDS limit above the 64 KiB default.  Done once per kernel
+// and device (the attribute call costs host time on every launch otherwise); KernelTag
+// is a type unique to the kernel instantiation, it only keys the bookkeeping.
+template <class KernelTag, class Kernel>
 hipError_t allow_lds(Kernel kernel, int bytes)
 {
     if (bytes <= 64 * 1024) return hipSuccess;
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    static std::atomic<unsigned long long> done{0};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const bool tracked = dev >= 0 && dev < 64;
+    if (tracked && ((done.load(std::memory_order_acquire) >> dev) & 1ull)) return hipSuccess;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess && tracked) done.fetch_or(1ull << dev, std::memory_order_release);
+    return e;
 }
+
+template <class S, int AF, int BF>
+struct TileKernelTag {};
+template <class S, int AF, int BF>
+struct PtileKernelTag {};
+template <class S, int AF, int BF>
+struct SkinnyKernelTag {};
 
 // out[i] = sum over the nsplit planes of ws, on `stream`
 hipError_t launch_reduce(const float *ws, float *out, size_t count, int nsplit, hipStream_t stream)
@@ -137,93 +157,91 @@ hipError_t launch_tile_shape(int m, int k, int n, const uint8_t *a, const uint8_
     const int nb = ((tiles_m + GM - 1) / GM) * ((tiles_n + GN - 1) / GN);
     const long grid = (long)((nb + 7) / 8) * 8 * GM * GN;
     auto kernel = gemm_tile_kernel<S, AF, BF>;
-    hipError_t e = allow_lds(kernel, S::LDS_BYTES);
+    hipError_t e = allow_lds<TileKernelTag<S, AF, BF>>(kernel, S::LDS_BYTES);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(S::THREADS), S::LDS_BYTES, stream,
                        m, k, n, a, b, out, tiles_m, tiles_n, GM, GN);
     return hipGetLastError();
 }
 
-// Super-block of GM x GN tiles that the CUs of one XCD work on together (at most 32
-// tiles, one per CU).  Chosen for: fewest rounds of the persistent walk; then the
-// smallest block, so that a problem with few tiles spreads over all eight XCDs (their
-// L2s and fabric links) instead of filling some and leaving others idle; then the
-// fewest operand panels per tile (1/GM + 1/GN), i.e. the most sharing inside the L2.
-struct TileBlocks {
-    int tiles_m, tiles_n, GM, GN, nb, rounds;
+// Work list of the persistent kernel for a tile shape: `bulk` tiles (a multiple of 256)
+// run as whole items, 256 per round; the remaining `tail` tiles are cut into nsplit K
+// slices each.  split_all cuts every tile (bulk = 0); otherwise only the tiles that do
+// not fill a round are cut.
+struct PtileWork {
+    int tiles_m, tiles_n, GM, bulk, tail, nsplit, rounds, slots;
+    bool ok;
 };
-TileBlocks tile_blocks(int m, int n, int bm, int bn, int nsplit)
+PtileWork ptile_work(int m, int n, int bm, int bn, int nsplit, bool split_all)
 {
-    TileBlocks t;
-    t.tiles_m = (m + bm - 1) / bm;
-    t.tiles_n = (n + bn - 1) / bn;
-    t.GM = t.GN = 1;
-    t.nb = t.tiles_m * t.tiles_n;
-    t.rounds = 0;
-    double best_share = 0.0;
-    for (int gm = 1; gm <= 8 && gm <= t.tiles_m; ++gm)
-        for (int gn = 1; gn <= 32 / gm && gn <= t.tiles_n; ++gn) {
-            const long nb = (long)((t.tiles_m + gm - 1) / gm) * ((t.tiles_n + gn - 1) / gn);
-            const long rounds = (nb * nsplit + 7) / 8;
-            if (rounds > 0x7fffffff) continue;
-            const double share = 1.0 / gm + 1.0 / gn;
-            const bool better = t.rounds == 0 || rounds < t.rounds ||
-                                (rounds == t.rounds && (gm * gn < t.GM * t.GN ||
-                                                        (gm * gn == t.GM * t.GN && share < best_share)));
-            if (better) {
-                t.GM = gm;
-                t.GN = gn;
-                t.nb = (int)nb;
-                t.rounds = (int)rounds;
-                best_share = share;
-            }
-        }
-    return t;
+    PtileWork w = {};
+    w.tiles_m = (m + bm - 1) / bm;
+    w.tiles_n = (n + bn - 1) / bn;
+    const long nt = (long)w.tiles_m * w.tiles_n;
+    w.ok = nt <= (1L << 30) / 16;
+    if (!w.ok) return w;
+    w.GM = w.tiles_m < 4 ? w.tiles_m : 4;
+    w.bulk = (split_all && nsplit > 1) ? 0 : (int)(nt / 256) * 256;
+    w.tail = (int)nt - w.bulk;
+    w.nsplit = w.tail > 0 ? nsplit : 1;
+    const long tail_items = (long)w.tail * w.nsplit;
+    w.rounds = w.bulk / 256 + (int)((tail_items + 255) / 256);
+    const long first_tail_round = tail_items < 256 ? tail_items : 256;
+    w.slots = w.bulk > 0 ? 32 : (int)((first_tail_round + 7) / 8);
+    return w;
 }
 
-// persistent form: one workgroup per CU walks the (tile, K slice) items of its XCD;
-// with nsplit > 1 the slices' partial sums go through the scratch buffer
+size_t ptile_scratch_bytes(const PtileWork &w, int bm, int bn)
+{
+    return w.nsplit > 1 ? (size_t)w.nsplit * w.tail * bm * bn * sizeof(float) : 0;
+}
+
+// persistent form: one workgroup per CU walks its share of the work list; the K slices'
+// partial sums go through the scratch buffer and a reduction pass
 template <class S, int AF, int BF>
 hipError_t launch_ptile_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
-                              int nsplit, int rotate, hipStream_t stream)
+                              int nsplit, bool split_all, int rotate, hipStream_t stream)
 {
     if (k % S::BK != 0 || nsplit < 1 || nsplit > k / S::BK) return hipErrorInvalidValue;
-    const TileBlocks t = tile_blocks(m, n, S::BM, S::BN, nsplit);
-    const int rounds = t.rounds;
-    const int grid = 8 * t.GM * t.GN;
-    float *dst = out;
-    if (nsplit > 1) {
-        void *ws = nullptr;
-        hipError_t e = scratch_get((size_t)nsplit * m * n * sizeof(float), &ws);
+    const PtileWork w = ptile_work(m, n, S::BM, S::BN, nsplit, split_all);
+    if (!w.ok) return hipErrorInvalidValue;
+    float *ws = nullptr;
+    if (w.nsplit > 1) {
+        void *p = nullptr;
+        hipError_t e = scratch_get(ptile_scratch_bytes(w, S::BM, S::BN), &p);
         if (e != hipSuccess) return e;
-        dst = static_cast<float *>(ws);
+        ws = static_cast<float *>(p);
     }
     auto kernel = gemm_ptile_kernel<S, AF, BF>;
-    hipError_t e = allow_lds(kernel, S::PTILE_LDS_BYTES);
+    hipError_t e = allow_lds<PtileKernelTag<S, AF, BF>>(kernel, S::PTILE_LDS_BYTES);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(S::THREADS), S::PTILE_LDS_BYTES, stream,
-                       m, k, n, a, b, dst, t.tiles_m, t.tiles_n, t.GM, t.GN, rounds, nsplit, rotate);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * w.slots)), dim3(S::THREADS), S::PTILE_LDS_BYTES, stream,
+                       m, k, n, a, b, out, ws, w.tiles_m, w.tiles_n, w.GM, w.bulk, w.tail, w.nsplit, w.rounds, rotate);
     e = hipGetLastError();
-    if (e != hipSuccess || nsplit == 1) return e;
-    return launch_reduce(dst, out, (size_t)m * n, nsplit, stream);
+    if (e != hipSuccess || w.nsplit == 1) return e;
+    const size_t threads = (size_t)w.tail * (S::BM * S::BN / 4);
+    hipLaunchKernelGGL(gemm_tile_slices_reduce_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream,
+                       ws, out, m, n, S::BM, S::BN, w.tiles_m, w.tiles_n, w.GM, w.bulk, w.tail, w.nsplit);
+    return hipGetLastError();
 }
 
 template <int AF, int BF>
 hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
-                       int variant, int nsplit, int rotate, hipStream_t stream)
+                       int variant, int nsplit, bool split_all, int rotate, hipStream_t stream)
 {
     const bool persistent = !(variant == 3 || variant == 4 || variant == 7);
     if (!persistent && nsplit != 1) return hipErrorInvalidValue;   // K slices only in the persistent kernels
     switch (variant) {
-    case 0: return launch_ptile_shape<TileP2, AF, BF>(m, k, n, a, b, out, nsplit, rotate, stream);
-    case 1: return launch_ptile_shape<TileP4, AF, BF>(m, k, n, a, b, out, nsplit, rotate, stream);
-    case 2: return launch_ptile_shape<TileP8, AF, BF>(m, k, n, a, b, out, nsplit, rotate, stream);
+    case 0: return launch_ptile_shape<TileP2, AF, BF>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
+    case 1: return launch_ptile_shape<TileP4, AF, BF>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
+    case 2: return launch_ptile_shape<TileP8, AF, BF>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
     case 3: return launch_tile_shape<TileS2, AF, BF>(m, k, n, a, b, out, stream);
     case 4: return launch_tile_shape<TileS4, AF, BF>(m, k, n, a, b, out, stream);
-    case 5: return launch_ptile_shape<TileH3, AF, BF>(m, k, n, a, b, out, nsplit, rotate, stream);
-    case 6: return launch_ptile_shape<TileQ2, AF, BF>(m, k, n, a, b, out, nsplit, rotate, stream);
+    case 5: return launch_ptile_shape<TileH3, AF, BF>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
+    case 6: return launch_ptile_shape<TileQ2, AF, BF>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
     case 7: return launch_tile_shape<TileS64, AF, BF>(m, k, n, a, b, out, stream);
-    case 8: return launch_ptile_shape<TileW3, AF, BF>(m, k, n, a, b, out, nsplit, rotate, stream);
+    case 8: return launch_ptile_shape<TileW3, AF, BF>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
+    case 9: return launch_ptile_shape<TileT2, AF, BF>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -249,7 +267,7 @@ hipError_t launch_skinny_shape(int m, int k, int n, const uint8_t *a, const uint
         dst = static_cast<float *>(ws);
     }
     auto kernel = gemm_skinny_kernel<S, AF, BF>;
-    hipError_t e = allow_lds(kernel, S::LDS_BYTES);
+    hipError_t e = allow_lds<SkinnyKernelTag<S, AF, BF>>(kernel, S::LDS_BYTES);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3((unsigned)(ngroups * nsplit)), dim3(64), S::LDS_BYTES, stream,
                        m, k, n, a, b, dst, ngroups, kchunk);
@@ -334,28 +352,31 @@ int select_algo(int m, int k, int n)
 // Which tiled kernel, how many K slices, which K-walk rotation.
 struct TilePlan {
     int variant, nsplit, rotate;
+    bool split_all;      // K slices for every tile (else only for the tiles that do not fill a round)
 };
 
 // Cost model behind the choice, in microseconds, fitted to MI355X timings of the
-// persistent kernels (operands cold in the caches, 128-byte K tiles; 30 shapes x 4 tile
-// shapes x 8 slice counts, the pick is within 1 % of the best measured candidate on
-// average):
-//   main kernel = max(rounds * (k_tiles_per_item * per_k_tile * load + per_item), input_bytes / stream_rate)
-//   load        = 0.6 + 0.4 * (share of the 256 CUs that have an item in a round): a chip
-//                 that is partly idle clocks higher and contends less for L2 and fabric
-//   K slices add one reduction pass over (nsplit + 1) planes of C.
-// rounds follows the kernel's own walk: 8 XCDs, each taking one super-block of tiles
-// per round.  The model only has to rank the candidates, not to predict the time.
+// persistent kernels (128-byte K tiles; 45 shapes x 5 tile shapes x 12 ways of cutting K;
+// the pick is within 1 % of the best measured candidate on average):
+//   a round of 256 whole tiles     = k_tiles * per_k_tile + per_item
+//   a round of tail items          = k_tiles_per_slice * per_k_tile * load + per_item
+//   load                           = 0.5 + 0.5 * (share of the 256 CUs with an item): a chip
+//                                    that is partly idle clocks higher and contends less
+//   main kernel                    = max(sum of rounds, input_bytes / stream_rate)
+//   K slices add one reduction pass over (nsplit + 1) x the cut tiles.
+// The model only has to rank the candidates, not to predict the time.
 struct PtileCost {
     int variant, bm, bn;
     double per_k_tile, per_item, stream_rate;   // us, us, bytes per us
 };
 constexpr PtileCost kPtileCosts[] = {
-    {0, 256, 256, 1.45, 11.0, 3.4e6},
-    {5, 128, 256, 0.95, 8.0, 5.0e6},
-    {6, 128, 128, 0.75, 2.5, 3.2e6},
-    {8, 256, 128, 0.90, 8.0, 4.0e6},
+    {0, 256, 256, 1.40, 13.0, 4.0e6},
+    {9, 192, 256, 1.25, 11.0, 4.6e6},
+    {5, 128, 256, 1.00, 8.0, 5.0e6},
+    {6, 128, 128, 0.75, 4.5, 3.2e6},
+    {8, 256, 128, 0.90, 10.0, 4.0e6},
 };
+constexpr double kIdleChipFactor = 0.5;
 constexpr int kSplitChoices[] = {1, 2, 3, 4, 6, 8, 12, 16};
 constexpr int kMinKTilesPerSlice = 12;
 constexpr size_t kMaxSplitScratch = (size_t)1 << 30;
@@ -364,7 +385,7 @@ TilePlan plan_tile(int m, int k, int n, int stages)
 {
     const long tiles256 = (long)((m + 255) / 256) * ((n + 255) / 256);
     const bool small = tiles256 < 192;
-    TilePlan best = {0, 1, 2};
+    TilePlan best = {0, 1, 2, false};
     if (k % 128 != 0) {                 // odd number of 64-byte K tiles
         best.variant = small ? 7 : 1;
         return best;
@@ -379,30 +400,50 @@ TilePlan plan_tile(int m, int k, int n, int stages)
         // the 256 x 128 tile pays off where it holds all rows of A at once (no second
         // row of tiles re-reading the same B rows) and is at least half full
         if (c.variant == 8 && (m <= 128 || m > 256)) continue;
-        for (int split : kSplitChoices) {
-            if (split > 1 && (kt / split < kMinKTilesPerSlice ||
-                              (size_t)split * m * n * sizeof(float) > kMaxSplitScratch))
-                continue;
-            const TileBlocks t = tile_blocks(m, n, c.bm, c.bn, split);
-            const int rounds = t.rounds;
-            const int kt_item = (kt + split - 1) / split;
-            double busy = (double)t.tiles_m * t.tiles_n * split / (256.0 * rounds);
-            if (busy > 1.0) busy = 1.0;
-            double cost = rounds * (kt_item * c.per_k_tile * (0.6 + 0.4 * busy) + c.per_item);
-            const double stream = ((double)m * k + (double)n * k) / c.stream_rate;
-            if (stream > cost) cost = stream;
-            if (split > 1) cost += 4.0 + (split + 1) * (double)m * n * 4.0 / 6.0e6;
-            if (cost < best_cost) {
-                best_cost = cost;
-                best.variant = c.variant;
-                best.nsplit = split;
+        for (int mode = 0; mode < 2; ++mode)          // 0: slices for the tail tiles only, 1: for all
+            for (int split : kSplitChoices) {
+                if (mode == 1 && split == 1) continue;      // same as mode 0
+                const PtileWork w = ptile_work(m, n, c.bm, c.bn, split, mode == 1);
+                if (!w.ok) continue;
+                if (split > 1 && (w.nsplit == 1 || kt / split < kMinKTilesPerSlice ||
+                                  ptile_scratch_bytes(w, c.bm, c.bn) > kMaxSplitScratch))
+                    continue;
+                // whole-tile rounds run with every CU busy; the rounds of tail items with
+                // whatever share of the CUs they fill
+                double cost = (w.bulk / 256) * (kt * c.per_k_tile + c.per_item);
+                const long tail_items = (long)w.tail * w.nsplit;
+                if (tail_items > 0) {
+                    const int tail_rounds = (int)((tail_items + 255) / 256);
+                    const double busy = (double)tail_items / (256.0 * tail_rounds);
+                    const int kt_item = (kt + w.nsplit - 1) / w.nsplit;
+                    cost += tail_rounds * (kt_item * c.per_k_tile * (kIdleChipFactor + (1.0 - kIdleChipFactor) * busy) + c.per_item);
+                }
+                const double stream = ((double)m * k + (double)n * k) / c.stream_rate;
+                if (stream > cost) cost = stream;
+                if (w.nsplit > 1) cost += 4.0 + (w.nsplit + 1) * (double)w.tail * c.bm * c.bn * 4.0 / 6.0e6;
+                if (cost < best_cost) {
+                    best_cost = cost;
+                    best.variant = c.variant;
+                    best.nsplit = w.nsplit;
+                    best.split_all = mode == 1;
+                }
             }
-        }
     }
     // K-walk rotation: per tile column while A is small enough to stay in an XCD's L2
-    // next to the B rows in flight, else per super-block
+    // next to the B rows in flight, else per XCD and round
     best.rotate = ((size_t)m * k <= ((size_t)2 << 20)) ? 1 : 2;
     return best;
+}
+
+size_t tile_plan_scratch_bytes(int m, int n, const TilePlan &p)
+{
+    if (p.nsplit <= 1) return 0;
+    for (const PtileCost &c : kPtileCosts)
+        if (c.variant == p.variant) {
+            const PtileWork w = ptile_work(m, n, c.bm, c.bn, p.nsplit, p.split_all);
+            return w.ok ? ptile_scratch_bytes(w, c.bm, c.bn) : 0;
+        }
+    return 0;
 }
 
 template <int AF, int BF>
@@ -429,9 +470,16 @@ hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, flo
             }
             p.variant = variant % 16;
             p.nsplit = 1;
+            p.split_all = false;
         }
-        if (nsplit > 0) p.nsplit = nsplit;
-        return launch_tile<AF, BF>(m, k, n, a, b, out, p.variant, p.nsplit, p.rotate, stream);
+        if (nsplit > 0) {          // forced: K slices for every tile
+            p.nsplit = nsplit;
+            p.split_all = true;
+        } else if (nsplit < 0) {   // forced: K slices for the tiles that do not fill a round
+            p.nsplit = -nsplit;
+            p.split_all = false;
+        }
+        return launch_tile<AF, BF>(m, k, n, a, b, out, p.variant, p.nsplit, p.split_all, p.rotate, stream);
     }
     case FP8GEMM_ALGO_SKINNY: {
         if (!aligned || !skinny_ok(m, k, n)) return hipErrorInvalidValue;
@@ -442,6 +490,7 @@ hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, flo
             if (variant / 16 > 0) p.tn = variant / 16;
         }
         if (nsplit > 0) p.nsplit = nsplit;
+        if (nsplit < 0) return hipErrorInvalidValue;
         return launch_skinny<AF, BF>(m, k, n, a, b, out, p, stream);
     }
     default:
@@ -527,7 +576,7 @@ int fp8gemm_plan(int m, int k, int n, int stages, int plan[4])
         const TilePlan p = plan_tile(m, k, n, stages);
         plan[1] = p.variant;
         plan[2] = p.nsplit;
-        plan[3] = p.rotate;
+        plan[3] = p.rotate + ((p.nsplit > 1 && !p.split_all) ? 16 : 0);
     }
     return 0;
 }
@@ -538,7 +587,7 @@ size_t fp8gemm_scratch_bytes(int m, int k, int n)
     int nsplit = 1;
     const int algo = select_algo(m, k, n);
     if (algo == FP8GEMM_ALGO_SKINNY) nsplit = plan_skinny(m, k, n).nsplit;
-    if (algo == FP8GEMM_ALGO_TILE) nsplit = plan_tile(m, k, n, 2).nsplit;
+    if (algo == FP8GEMM_ALGO_TILE) return tile_plan_scratch_bytes(m, n, plan_tile(m, k, n, 2));
     return nsplit > 1 ? (size_t)nsplit * m * n * sizeof(float) : 0;
 }
 

@@ -1,8 +1,8 @@
 // Persistent LDS-tiled MFMA kernel for compute-bound shapes.
 //
-// The grid is one workgroup per CU; every workgroup walks a list of BM x BN
-// tiles of C.  Inside a tile the K loop is a software pipeline with three
-// levels, all of them explicit:
+// The grid is one workgroup per CU; every workgroup walks a list of work items,
+// each a BM x BN tile of C over all of K or over one slice of K.  Inside an item
+// the K loop is a software pipeline with three levels, all of them explicit:
 //   * global -> LDS: 128-bit buffer loads that write LDS directly
 //     (buffer_load_dwordx4 ... lds) into a ring of STAGES buffers, issued
 //     STAGES-1 K tiles ahead of their use; no registers involved;
@@ -73,8 +73,10 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                                                                  const uint8_t *__restrict__ A,
                                                                  const uint8_t *__restrict__ B,
                                                                  float *__restrict__ C,
-                                                                 int tiles_m, int tiles_n, int GM, int GN,
-                                                                 int rounds, int nsplit, int rotate)
+                                                                 float *__restrict__ ws,
+                                                                 int tiles_m, int tiles_n, int GM,
+                                                                 int bulk, int tail, int nsplit,
+                                                                 int rounds, int rotate)
 {
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, CH = S::CH, RPI = S::RPI;
     constexpr int STAGES = S::STAGES, TM = S::TM, TN = S::TN, KSTEPS = S::KSTEPS;
@@ -104,28 +106,60 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
     const uint32_t b_base = (uint32_t)(BM * BK) + (uint32_t)(wn * (BN / S::WN) + fi) * BK;
     const int KT = K / BK;                         // K tiles of the whole problem
 
-    // Work items are (super-block of tiles, K slice): with nsplit > 1 the K tiles are cut
-    // into nsplit contiguous slices and slice s writes its partial sums to the s-th M x N
-    // plane behind C (the host adds the planes up afterwards).  Workgroups with equal id
-    // mod 8 share an XCD (and its L2): XCD x takes the items x*rounds .. x*rounds+rounds-1,
-    // slot q of its 32 workgroups takes tile q of each item's super-block.
+    // Work items.  The tiles of C are numbered along strips of GM tile rows (down a
+    // column of the strip first, then on to the next column), so that consecutive tile
+    // numbers form compact GM-row windows.  The first `bulk` tiles (a multiple of 256)
+    // are items of their own, 256 per round: XCD x takes 32 consecutive ones, one per
+    // CU, and shares their operand panels in its L2 (workgroups with equal id mod 8 sit
+    // on one XCD).  The last `tail` tiles, too few to fill a round, are cut into nsplit
+    // K slices each (slice-major item order: neighbours are still neighbouring tiles);
+    // every round of such items is spread evenly over the eight XCDs.  Slice s of tail
+    // tile u writes its partial sums to slot s*tail + u of the scratch `ws` (BM x BN
+    // floats, row stride BN; the host adds the slices up afterwards); unsplit items
+    // write C directly.
     const int xcd = blockIdx.x & 7;
     const int slot = blockIdx.x >> 3;
-    const int nb_n = (tiles_n + GN - 1) / GN;
-    const int nb_mn = ((tiles_m + GM - 1) / GM) * nb_n;
-    const int nb_total = nb_mn * nsplit;
+    const int bulk_rounds = bulk >> 8;
+    const int tail_items = tail * nsplit;
 
-    // tile and K-tile range [kt0, kt0 + T) of round r; false when there is none
-    auto tile_of_round = [&](int r, int &tm, int &tn, int &slice, int &kt0, int &T) -> bool {
-        const int item = xcd * rounds + r;
-        if (r >= rounds || item >= nb_total || slot >= GM * GN) return false;
-        slice = item / nb_mn;
-        const int blk = item - slice * nb_mn;
-        tm = (blk / nb_n) * GM + slot / GN;
-        tn = (blk % nb_n) * GN + slot % GN;
-        kt0 = (int)((long)KT * slice / nsplit);
-        T = (int)((long)KT * (slice + 1) / nsplit) - kt0;
-        return tm < tiles_m && tn < tiles_n;
+    // item of round r: tile, slice, K-tile range [kt0, kt0 + T), scratch slot (-1: writes C);
+    // false when this workgroup has none
+    auto tile_of_round = [&](int r, int &tm, int &tn, int &kt0, int &T, int &ws_slot) -> bool {
+        if (r >= rounds) return false;
+        int g, slice = 0;
+        ws_slot = -1;
+        if (r < bulk_rounds) {
+            if (slot >= 32) return false;
+            g = r * 256 + xcd * 32 + slot;
+        } else {
+            const int first = (r - bulk_rounds) * 256;
+            int count = tail_items - first;
+            count = count > 256 ? 256 : count;
+            if (count <= 0) return false;
+            const int per_xcd = (count + 7) >> 3;
+            const int local = xcd * per_xcd + slot;
+            if (slot >= per_xcd || local >= count) return false;
+            const int u = first + local;
+            slice = u / tail;
+            const int t = u - slice * tail;
+            g = bulk + t;
+            if (nsplit > 1) ws_slot = slice * tail + t;
+        }
+        const int per_strip = GM * tiles_n;
+        const int strip = g / per_strip;
+        const int rem = g - strip * per_strip;
+        int h = tiles_m - strip * GM;
+        h = h > GM ? GM : h;
+        const int col = rem / h;
+        // (the divisions may run on the vector unit; every lane holds the same values)
+        tn = __builtin_amdgcn_readfirstlane(col);
+        tm = __builtin_amdgcn_readfirstlane(strip * GM + rem - col * h);
+        const int split = r < bulk_rounds ? 1 : nsplit;
+        const int k0 = (int)((long)KT * slice / split);
+        kt0 = __builtin_amdgcn_readfirstlane(k0);
+        T = __builtin_amdgcn_readfirstlane((int)((long)KT * (slice + 1) / split) - k0);
+        ws_slot = __builtin_amdgcn_readfirstlane(ws_slot);
+        return true;
     };
 
     // Global -> LDS load plan: one buffer resource per operand and tile (base =
@@ -151,7 +185,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
     // power-of-two K those are the bits that select the HBM channel, so the whole chip
     // would queue on a few channels at a time.  rotate == 1 starts every tile column at
     // its own K tile (the workgroups of a column still share their B rows through L2; A
-    // must then be small enough to stay in L2), rotate == 2 every super-block (all
+    // must then be small enough to stay in L2), rotate == 2 every XCD in every round (all
     // sharing inside an XCD is kept), 0 leaves the walk alone.
     int kt_base = 0, kt_rot = 0, kt_count = 1;
     auto plan_loads = [&](int tile_m, int tile_n, int kt0, int count, int item) {
@@ -160,7 +194,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         rsB = make_buffer_resource(B + (size_t)n0 * K, (unsigned long long)(N - n0) * (unsigned long long)K);
         kt_base = kt0;
         kt_count = count;
-        const unsigned key = rotate == 1 ? (unsigned)tile_n : (unsigned)item;
+        const unsigned key = rotate == 1 ? (unsigned)tile_n : (unsigned)item;   // item: (round, XCD)
         // (the division runs on the vector unit; the result is the same in every lane)
         kt_rot = rotate == 0 ? 0 : __builtin_amdgcn_readfirstlane((int)(((key * 2654435761u) >> 8) % (unsigned)count));
     };
@@ -180,10 +214,10 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         for (int j = 0; j < S::LOADS; ++j) issue_load(j, ktile, stage);
     };
 
-    int tile_m = 0, tile_n = 0, slice = 0, kt0 = 0, T = 0;
-    bool have = tile_of_round(0, tile_m, tile_n, slice, kt0, T);
+    int tile_m = 0, tile_n = 0, kt0 = 0, T = 0, ws_slot = -1;
+    bool have = tile_of_round(0, tile_m, tile_n, kt0, T, ws_slot);
     if (have) {
-        plan_loads(tile_m, tile_n, kt0, T, xcd * rounds + 0);
+        plan_loads(tile_m, tile_n, kt0, T, xcd);
 #pragma unroll
         for (int t = 0; t < STAGES - 1; ++t)
             if (t < T) issue_all_loads(t, t);
@@ -192,9 +226,9 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
     for (int r = 0; r < rounds; ++r) {
         if (!have) {
             // nothing here this round; still look at the next one
-            have = tile_of_round(r + 1, tile_m, tile_n, slice, kt0, T);
+            have = tile_of_round(r + 1, tile_m, tile_n, kt0, T, ws_slot);
             if (have) {
-                plan_loads(tile_m, tile_n, kt0, T, xcd * rounds + r + 1);
+                plan_loads(tile_m, tile_n, kt0, T, (r + 1) * 8 + xcd);
 #pragma unroll
                 for (int t = 0; t < STAGES - 1; ++t)
                     if (t < T) issue_all_loads(t, t);
@@ -202,7 +236,6 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
             continue;
         }
         const int m0 = tile_m * BM, n0 = tile_n * BN;
-        float *__restrict__ Cout = C + (size_t)slice * ((size_t)M * (size_t)N);
 
         v16f acc[TM][TN];
 #pragma unroll
@@ -318,10 +351,10 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         // all waves are done reading LDS for this tile before the ring is reused
         wait_lgkmcnt0();
         __syncthreads();
-        int next_m = 0, next_n = 0, next_slice = 0, next_kt0 = 0, next_T = 0;
-        have = tile_of_round(r + 1, next_m, next_n, next_slice, next_kt0, next_T);
+        int next_m = 0, next_n = 0, next_kt0 = 0, next_T = 0, next_ws_slot = -1;
+        have = tile_of_round(r + 1, next_m, next_n, next_kt0, next_T, next_ws_slot);
         if (have) {
-            plan_loads(next_m, next_n, next_kt0, next_T, xcd * rounds + r + 1);
+            plan_loads(next_m, next_n, next_kt0, next_T, (r + 1) * 8 + xcd);
 #pragma unroll
             for (int t = 0; t < STAGES - 1; ++t)
                 if (t < next_T) issue_all_loads(t, t);
@@ -331,8 +364,14 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         // register q of lane (fi, fg) holds C[row0 + fi][col0 + 8*(q/4) + 4*fg + q%4]
         const int wrow0 = m0 + wm * (BM / S::WM);
         const int wcol0 = n0 + wn * (BN / S::WN);
-        const bool full = (m0 + BM <= M) && (n0 + BN <= N) && (N % 4 == 0) &&
-                          (reinterpret_cast<uintptr_t>(Cout) % 16 == 0);
+        // destination of this item: its tile of C (row stride N), or a whole BM x BN slot of
+        // the scratch (row stride BN; rows and columns past the matrix hold zeros)
+        const bool to_ws = ws_slot >= 0;
+        float *__restrict__ tile_out = to_ws ? ws + (size_t)ws_slot * (size_t)(BM * BN)
+                                             : C + (size_t)m0 * (size_t)N + n0;
+        const size_t ldo = to_ws ? (size_t)BN : (size_t)N;
+        const bool full = to_ws || ((m0 + BM <= M) && (n0 + BN <= N) && (N % 4 == 0) &&
+                                    (reinterpret_cast<uintptr_t>(C) % 16 == 0));
         if (full) {
             // Each wave transposes its results through a private strip of LDS (the part of
             // the ring the next tile's first loads do not use, plus the LDS above the ring)
@@ -359,7 +398,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
 #pragma unroll
                     for (int r0 = 0; r0 < 32; r0 += RPI_ST) {
                         const v4f v = *reinterpret_cast<const v4f *>(stg + (r0 + rl) * ROWB + cl * 16);
-                        float *dst = Cout + (size_t)(wrow0 + i * 32 + r0 + rl) * N + wcol0 + c0 + cl * 4;
+                        float *dst = tile_out + (size_t)(wrow0 - m0 + i * 32 + r0 + rl) * ldo + (wcol0 - n0 + c0 + cl * 4);
                         *reinterpret_cast<v4f *>(dst) = v;
                     }
                 }
@@ -373,16 +412,16 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
 #pragma unroll
                         for (int q = 0; q < 16; ++q) {
                             const int col = wcol0 + j * 32 + 8 * (q >> 2) + 4 * fg + (q & 3);
-                            if (col < N) Cout[(size_t)row * N + col] = acc[i][j][q];
+                            if (col < N) C[(size_t)row * N + col] = acc[i][j][q];
                         }
                 }
             }
         }
         tile_m = next_m;
         tile_n = next_n;
-        slice = next_slice;
         kt0 = next_kt0;
         T = next_T;
+        ws_slot = next_ws_slot;
     }
 }
 

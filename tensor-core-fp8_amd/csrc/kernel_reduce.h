@@ -36,4 +36,50 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce4_kernel(const v4f *__r
     C[i] = s;
 }
 
+// Partial sums of the persistent tiled kernel: scratch slot s*tail + u holds slice s of
+// tail tile u as BM x BN floats (row stride BN).  One thread per 4 consecutive columns
+// of a tile adds the slices in ascending order and writes the part that lies inside C.
+// The tile numbering is the kernel's: strips of GM tile rows, down a column first.
+__global__ __launch_bounds__(256) void gemm_tile_slices_reduce_kernel(const float *__restrict__ ws,
+                                                                      float *__restrict__ C, int M, int N,
+                                                                      int BM, int BN, int tiles_m, int tiles_n,
+                                                                      int GM, int bulk, int tail, int nsplit)
+{
+    const int quads_per_tile = BM * BN / 4;
+    const size_t id = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int u = (int)(id / quads_per_tile);
+    if (u >= tail) return;
+    const int q = (int)(id - (size_t)u * quads_per_tile);
+    const int row = q / (BN / 4);
+    const int col = (q - row * (BN / 4)) * 4;
+    const int g = bulk + u;
+    const int per_strip = GM * tiles_n;
+    const int strip = g / per_strip;
+    const int rem = g - strip * per_strip;
+    int h = tiles_m - strip * GM;
+    h = h > GM ? GM : h;
+    const int tn = rem / h;
+    const int tm = strip * GM + rem - tn * h;
+    const int grow = tm * BM + row;
+    const int gcol = tn * BN + col;
+    if (grow >= M || gcol >= N) return;
+    const size_t tile_floats = (size_t)BM * BN;
+    const float *src = ws + (size_t)u * tile_floats + (size_t)row * BN + col;
+    v4f s = *reinterpret_cast<const v4f *>(src);
+    for (int p = 1; p < nsplit; ++p) {
+        const v4f v = *reinterpret_cast<const v4f *>(src + (size_t)p * tail * tile_floats);
+        s[0] += v[0];
+        s[1] += v[1];
+        s[2] += v[2];
+        s[3] += v[3];
+    }
+    float *dst = C + (size_t)grow * N + gcol;
+    if (gcol + 3 < N && N % 4 == 0 && reinterpret_cast<uintptr_t>(C) % 16 == 0) {
+        *reinterpret_cast<v4f *>(dst) = s;
+    } else {
+        for (int e = 0; e < 4; ++e)
+            if (gcol + e < N) dst[e] = s[e];
+    }
+}
+
 #endif  // FP8GEMM_KERNEL_REDUCE_H

@@ -69,15 +69,19 @@ def test_kernel_selection_is_pure_host_logic(pkg):
     fam, var, slices, _ = pkg.plan(256, 28672, 8192)
     assert fam == pkg.ALGO_TILE and slices > 1
     assert pkg.plan(100, 100, 100)[0] == pkg.ALGO_DIRECT
-    for shape in [(256, 28672, 8192), (64, 28672, 8192), (300, 4096, 500), (8192, 8192, 8192)]:
+    for shape in [(256, 28672, 8192), (64, 28672, 8192), (300, 4096, 500), (8192, 8192, 8192), (4352, 4352, 4352)]:
         slices = pkg.plan(*shape)[2]
-        want = slices * shape[0] * shape[2] * 4 if slices > 1 else 0
-        assert L.fp8gemm_scratch_bytes(*shape) == want
+        assert (L.fp8gemm_scratch_bytes(*shape) > 0) == (slices > 1)
+    assert L.fp8gemm_scratch_bytes(64, 28672, 8192) == pkg.plan(64, 28672, 8192)[2] * 64 * 8192 * 4
+    # 17 x 17 tiles of 256 x 256: one round of whole tiles, the 33 left over cut into K slices
+    fam, var, slices, mode = pkg.plan(4352, 4352, 4352)
+    assert fam == pkg.ALGO_TILE and slices > 1 and mode >= 16
+    assert L.fp8gemm_scratch_bytes(4352, 4352, 4352) == slices * 33 * 256 * 256 * 4
     out = (ctypes.c_int * 4)()
     assert L.fp8gemm_plan(0, 1, 1, 2, out) == 1 and L.fp8gemm_plan(1, 1, 1, 3, out) == 1
     # few tiles and a long K: the tiled kernels cut K into slices, whole planes of partial sums
     s = L.fp8gemm_scratch_bytes(256, 28672, 8192)
-    assert s >= 2 * 256 * 8192 * 4 and s % (256 * 8192 * 4) == 0
+    assert s >= 2 * 256 * 8192 * 4 and s % (128 * 128 * 4) == 0
 
 
 def test_generators_are_reproducible_and_counter_based(pkg):

@@ -107,7 +107,7 @@ def test_normal_inputs_within_fp32_reordering_bound(pkg, oracle, fa, fb, algo, s
     assert worst < 0.25
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9])
 @pytest.mark.parametrize("shape", [(256, 256, 256), (300, 512, 200), (1000, 1024, 900), (513, 384, 257), (64, 128, 2048)])
 def test_every_tile_variant(pkg, oracle, variant, shape):
     """Each compiled shape of the tiled kernels (persistent and one-tile-per-workgroup),
@@ -132,6 +132,28 @@ def test_tile_k_slices(pkg, oracle, variant, split, shape):
     C = run_gpu(pkg, A, 1, B, 0, algo=ALGOS["tile"], variant=variant, split_k=split)
     worst = assert_within_bound(oracle, C, A, 1, B, 0)
     assert worst < 0.25
+
+
+@pytest.mark.parametrize("variant,split,shape", [
+    (6, -3, (2200, 2048, 2300)),      # 18 x 18 tiles of 128 x 128: 256 whole items + 68 tail tiles in 3 slices
+    (6, -2, (2304, 1024, 2304)),
+    (5, -4, (2100, 1536, 4500)),      # 17 x 18 tiles of 128 x 256
+    (0, -2, (4200, 1024, 4300)),      # 17 x 17 tiles of 256 x 256
+    (8, -5, (4352, 1280, 2200)),      # 17 x 18 tiles of 256 x 128
+    (1, -2, (4352, 1088, 4352)),      # 64-byte K tiles, 17 of them
+])
+def test_tile_k_slices_for_the_last_partial_round(pkg, oracle, variant, split, shape):
+    """More tiles than CUs: the rounds of 256 whole tiles write C directly, the tiles left
+    over are cut into K slices that go through the scratch and the reduction kernel."""
+    M, K, N = shape
+    A = pkg.fill((M, K), 0, seed=0xA11CE + K - split, dist="normal", sigma=4.0)
+    B = pkg.fill((N, K), 1, seed=0xB0B + K - split, dist="normal", sigma=4.0)
+    C = run_gpu(pkg, A, 0, B, 1, algo=ALGOS["tile"], variant=variant, split_k=split)
+    rows = np.arange(0, M, 5, dtype=np.int32)
+    worst = assert_within_bound(oracle, C, A, 0, B, 1, rows=rows)
+    assert worst < 0.25
+    # every element was written (the NaN fill is gone), the leftover tiles included
+    assert np.isfinite(C).all()
 
 
 @pytest.mark.parametrize("variant", [1, 7, None])
