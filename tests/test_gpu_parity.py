@@ -240,3 +240,49 @@ def test_small_integers_are_exact(pkg, oracle, algo, shape):
     assert np.array_equal(C, Cref)
     ints = oracle.decode(A, 0).astype(np.int64) @ oracle.decode(B, 1).astype(np.int64).T
     assert np.array_equal(C.astype(np.int64), ints)
+
+
+def test_scratch_grows_and_is_reused_across_calls_and_streams(pkg, oracle):
+    """Calls that need the partial-sum scratch, in growing and shrinking order, on the default
+    stream and on a side stream (ordered by the caller): every result is right, before and
+    after the scratch has been reallocated."""
+    import torch
+    shapes = [(256, 8192, 1024), (256, 8192, 2048), (256, 8192, 1024), (300, 6144, 1000), (256, 8192, 2048)]
+    side = torch.cuda.Stream()
+    need = [pkg.lib().fp8gemm_scratch_bytes(*s) for s in shapes]
+    assert need[0] > 0 and need[1] > need[0]           # the second call has to grow the buffer
+    for idx, (M, K, N) in enumerate(shapes):
+        A = pkg.fill((M, K), 0, seed=0xA11CE + 100 + idx, dist="normal", sigma=4.0)
+        B = pkg.fill((N, K), 0, seed=0xB0B + 100 + idx, dist="normal", sigma=4.0)
+        dA = torch.from_numpy(A).cuda()
+        dB = torch.from_numpy(B).cuda()
+        out = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()
+        if idx % 2:
+            with torch.cuda.stream(side):
+                pkg.gemm(dA, dB, out=out, a_fmt=0, b_fmt=0, stream=side)
+            side.synchronize()
+        else:
+            pkg.gemm(dA, dB, out=out, a_fmt=0, b_fmt=0)
+            torch.cuda.synchronize()
+        worst = assert_within_bound(oracle, out.cpu().numpy(), A, 0, B, 0)
+        assert worst < 0.25, (idx, worst)
+
+
+def test_back_to_back_launches_without_synchronisation(pkg, oracle):
+    """Twenty launches of alternating shapes queued on one stream with no host
+    synchronisation in between (stream order is the only ordering): each output is right."""
+    import torch
+    cases = []
+    for idx in range(20):
+        M, K, N = [(16, 2048, 1024), (512, 1024, 768), (256, 8192, 1024), (1, 4096, 256)][idx % 4]
+        A = pkg.fill((M, K), idx % 2, seed=0xA11CE + 200 + idx, dist="normal", sigma=2.0)
+        B = pkg.fill((N, K), 0, seed=0xB0B + 200 + idx, dist="normal", sigma=2.0)
+        cases.append((A, B, torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(),
+                      torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda"), idx % 2))
+    torch.cuda.synchronize()
+    for A, B, dA, dB, out, fa in cases:
+        pkg.gemm(dA, dB, out=out, a_fmt=fa, b_fmt=0)
+    torch.cuda.synchronize()
+    for A, B, dA, dB, out, fa in cases:
+        assert_within_bound(oracle, out.cpu().numpy(), A, fa, B, 0)
