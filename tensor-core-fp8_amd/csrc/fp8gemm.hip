@@ -107,7 +107,7 @@ hipError_t allow_lds(Kernel kernel, int bytes)
 
 template <class S, int AF, int BF>
 struct TileKernelTag {};
-template <class S, int AF, int BF>
+template <class S, int AF, int BF, bool KOVER>
 struct PtileKernelTag {};
 template <class S, int AF, int BF>
 struct SkinnyKernelTag {};
@@ -198,11 +198,11 @@ size_t ptile_scratch_bytes(const PtileWork &w, int bm, int bn)
 
 // persistent form: one workgroup per CU walks its share of the work list; the K slices'
 // partial sums go through the scratch buffer and a reduction pass
-template <class S, int AF, int BF>
-hipError_t launch_ptile_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
-                              int nsplit, bool split_all, int rotate, hipStream_t stream)
+template <class S, int AF, int BF, bool KOVER>
+hipError_t launch_ptile_shape_k(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
+                                int nsplit, bool split_all, int rotate, hipStream_t stream)
 {
-    if (k % S::BK != 0 || nsplit < 1 || nsplit > k / S::BK) return hipErrorInvalidValue;
+    if (k % 16 != 0 || k > (1 << 23) || nsplit < 1 || nsplit > (k + S::BK - 1) / S::BK) return hipErrorInvalidValue;
     const PtileWork w = ptile_work(m, n, S::BM, S::BN, nsplit, split_all);
     if (!w.ok) return hipErrorInvalidValue;
     float *ws = nullptr;
@@ -212,8 +212,8 @@ hipError_t launch_ptile_shape(int m, int k, int n, const uint8_t *a, const uint8
         if (e != hipSuccess) return e;
         ws = static_cast<float *>(p);
     }
-    auto kernel = gemm_ptile_kernel<S, AF, BF>;
-    hipError_t e = allow_lds<PtileKernelTag<S, AF, BF>>(kernel, S::PTILE_LDS_BYTES);
+    auto kernel = gemm_ptile_kernel<S, AF, BF, KOVER>;
+    hipError_t e = allow_lds<PtileKernelTag<S, AF, BF, KOVER>>(kernel, S::PTILE_LDS_BYTES);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * w.slots)), dim3(S::THREADS), S::PTILE_LDS_BYTES, stream,
                        m, k, n, a, b, out, ws, w.tiles_m, w.tiles_n, w.GM, w.bulk, w.tail, w.nsplit, w.rounds, rotate);
@@ -225,6 +225,19 @@ hipError_t launch_ptile_shape(int m, int k, int n, const uint8_t *a, const uint8
     return hipGetLastError();
 }
 
+// OVERHANG_TOO: this shape is also compiled for a K that is not a multiple of its K tile
+template <class S, int AF, int BF, bool OVERHANG_TOO>
+hipError_t launch_ptile_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
+                              int nsplit, bool split_all, int rotate, hipStream_t stream)
+{
+    if (k % S::BK == 0)
+        return launch_ptile_shape_k<S, AF, BF, false>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
+    if constexpr (OVERHANG_TOO)
+        return launch_ptile_shape_k<S, AF, BF, true>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
+    else
+        return hipErrorInvalidValue;
+}
+
 template <int AF, int BF>
 hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
                        int variant, int nsplit, bool split_all, int rotate, hipStream_t stream)
@@ -232,16 +245,16 @@ hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, 
     const bool persistent = !(variant == 3 || variant == 4 || variant == 7);
     if (!persistent && nsplit != 1) return hipErrorInvalidValue;   // K slices only in the persistent kernels
     switch (variant) {
-    case 0: return launch_ptile_shape<TileP2, AF, BF>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
-    case 1: return launch_ptile_shape<TileP4, AF, BF>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
-    case 2: return launch_ptile_shape<TileP8, AF, BF>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
+    case 0: return launch_ptile_shape<TileP2, AF, BF, true>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
+    case 1: return launch_ptile_shape<TileP4, AF, BF, true>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
+    case 2: return launch_ptile_shape<TileP8, AF, BF, false>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
     case 3: return launch_tile_shape<TileS2, AF, BF>(m, k, n, a, b, out, stream);
     case 4: return launch_tile_shape<TileS4, AF, BF>(m, k, n, a, b, out, stream);
-    case 5: return launch_ptile_shape<TileH3, AF, BF>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
-    case 6: return launch_ptile_shape<TileQ2, AF, BF>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
+    case 5: return launch_ptile_shape<TileH3, AF, BF, true>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
+    case 6: return launch_ptile_shape<TileQ2, AF, BF, true>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
     case 7: return launch_tile_shape<TileS64, AF, BF>(m, k, n, a, b, out, stream);
-    case 8: return launch_ptile_shape<TileW3, AF, BF>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
-    case 9: return launch_ptile_shape<TileT2, AF, BF>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
+    case 8: return launch_ptile_shape<TileW3, AF, BF, false>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
+    case 9: return launch_ptile_shape<TileT2, AF, BF, false>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -345,7 +358,7 @@ SkinnyPlan plan_skinny(int m, int k, int n)
 int select_algo(int m, int k, int n)
 {
     if (skinny_ok(m, k, n)) return FP8GEMM_ALGO_SKINNY;
-    if (k % 64 == 0) return FP8GEMM_ALGO_TILE;
+    if (k % 16 == 0 && k <= (1 << 23)) return FP8GEMM_ALGO_TILE;
     return FP8GEMM_ALGO_DIRECT;
 }
 
@@ -386,20 +399,18 @@ TilePlan plan_tile(int m, int k, int n, int stages)
     const long tiles256 = (long)((m + 255) / 256) * ((n + 255) / 256);
     const bool small = tiles256 < 192;
     TilePlan best = {0, 1, 2, false};
-    if (k % 128 != 0) {                 // odd number of 64-byte K tiles
-        best.variant = small ? 7 : 1;
-        return best;
-    }
     if (stages == 4) {                  // the 4-deep rings: one shape for big problems, one for small
-        best.variant = small ? 4 : 1;
+        best.variant = (small && k % 128 == 0) ? 4 : 1;       // (the small one needs whole 128-byte K tiles)
         return best;
     }
-    const int kt = k / 128;
+    const int kt = (k + 127) / 128;
     double best_cost = 1e30;
     for (const PtileCost &c : kPtileCosts) {
         // the 256 x 128 tile pays off where it holds all rows of A at once (no second
         // row of tiles re-reading the same B rows) and is at least half full
         if (c.variant == 8 && (m <= 128 || m > 256)) continue;
+        // a K that is not a multiple of 128: only the shapes compiled for an overhanging K tile
+        if (k % 128 != 0 && !(c.variant == 0 || c.variant == 5 || c.variant == 6)) continue;
         for (int mode = 0; mode < 2; ++mode)          // 0: slices for the tail tiles only, 1: for all
             for (int split : kSplitChoices) {
                 if (mode == 1 && split == 1) continue;      // same as mode 0
@@ -459,7 +470,7 @@ hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, flo
     case FP8GEMM_ALGO_DIRECT:
         return launch_direct<AF, BF>(m, k, n, a, b, out, stream);
     case FP8GEMM_ALGO_TILE: {
-        if (!aligned || k % 64 != 0) return hipErrorInvalidValue;
+        if (!aligned || k % 16 != 0 || k > (1 << 23)) return hipErrorInvalidValue;
         TilePlan p = plan_tile(m, k, n, stages);
         if (variant >= 0) {
             // tuning hook: variant = shape index + 16 * (1 + K-walk rotation mode); a bare

@@ -23,7 +23,8 @@
 // turns the epilogue into 128-bit stores.
 //
 // LDS layout, swizzle and the K-permutation freedom are as in kernel_tile.h.
-// Requirements checked by the host: K % BK == 0, 16-byte aligned a and b.
+// Requirements checked by the host: K % 16 == 0 (rows start 16-byte aligned and a
+// 16-byte chunk never straddles the end of a row), K < 2^23, 16-byte aligned a and b.
 #ifndef FP8GEMM_KERNEL_PTILE_H
 #define FP8GEMM_KERNEL_PTILE_H
 
@@ -40,6 +41,10 @@ __device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xC
 // Written as inline assembly so that the compiler does not order it against the
 // fragment reads (they never touch the ring slot being filled; the barrier
 // protocol guarantees it).  Completion is tracked with wait_vmcnt by hand.
+// M0 (the LDS base of the load) is named as clobbered so that the compiler keeps nothing
+// in it across the statement; it warns that M0 is a reserved register, which is the point.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void buffer_load_lds_b128(v4i rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff)
 {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
@@ -47,6 +52,7 @@ __device__ __forceinline__ void buffer_load_lds_b128(v4i rsrc, uint32_t lds_addr
                  : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
                  : "m0");
 }
+#pragma clang diagnostic pop
 
 // 16-byte-per-lane LDS store whose data operand stays in accumulation registers
 // (the MFMA results live there; copying all of them to ordinary vector registers
@@ -68,7 +74,9 @@ __device__ __forceinline__ v4i make_buffer_resource(const void *base, unsigned l
     return r;
 }
 
-template <class S, int AF, int BF>
+// KOVER: the last K tile may overhang K (K % BK != 0); compiled separately so that the
+// common case carries no test for it.
+template <class S, int AF, int BF, bool KOVER>
 __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, int N,
                                                                  const uint8_t *__restrict__ A,
                                                                  const uint8_t *__restrict__ B,
@@ -104,7 +112,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         for (int j = 0; j < 2; ++j) frag_off[s][j] = (uint32_t)(((s * 4 + 2 * fg + j) ^ sw) * 16);
     const uint32_t a_base = (uint32_t)(wm * (BM / S::WM) + fi) * BK;
     const uint32_t b_base = (uint32_t)(BM * BK) + (uint32_t)(wn * (BN / S::WN) + fi) * BK;
-    const int KT = K / BK;                         // K tiles of the whole problem
+    const int KT = (K + BK - 1) / BK;              // K tiles of the whole problem; the last may overhang K
 
     // Work items.  The tiles of C are numbered along strips of GM tile rows (down a
     // column of the strip first, then on to the next column), so that consecutive tile
@@ -163,11 +171,12 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
     };
 
     // Global -> LDS load plan: one buffer resource per operand and tile (base =
-    // first row of the tile, extent = what is left of the matrix), a
-    // loop-invariant 32-bit offset per load (row * K + chunk * 16) and a uniform
-    // offset that walks K.  Rows past the end of the matrix fall outside the
-    // extent and read as zero bytes (fp8 +0.0), which is how tiles that overhang
-    // m or n are handled.
+    // first row of the tile, extent = the tile's rows that exist), a loop-invariant
+    // 32-bit offset per load (row * K + chunk * 16) and a uniform offset that walks K.
+    // Rows past the end of the matrix fall outside the extent and read as zero bytes
+    // (fp8 +0.0), which is how tiles that overhang m or n are handled; in the K tile
+    // that overhangs K, the chunks past the end of a row are sent outside the extent
+    // on purpose (they would otherwise read the next row).
     uint32_t ld_off[S::LOADS];
 #pragma unroll
     for (int j = 0; j < S::LOADS; ++j) {
@@ -188,10 +197,12 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
     // must then be small enough to stay in L2), rotate == 2 every XCD in every round (all
     // sharing inside an XCD is kept), 0 leaves the walk alone.
     int kt_base = 0, kt_rot = 0, kt_count = 1;
-    auto plan_loads = [&](int tile_m, int tile_n, int kt0, int count, int item) {
+    auto plan_loads = [&](int tile_m, int tile_n, int kt0, int count, int item) __attribute__((always_inline)) {
         const int m0 = tile_m * BM, n0 = tile_n * BN;
-        rsA = make_buffer_resource(A + (size_t)m0 * K, (unsigned long long)(M - m0) * (unsigned long long)K);
-        rsB = make_buffer_resource(B + (size_t)n0 * K, (unsigned long long)(N - n0) * (unsigned long long)K);
+        const int rows_a = M - m0 < BM ? M - m0 : BM;
+        const int rows_b = N - n0 < BN ? N - n0 : BN;
+        rsA = make_buffer_resource(A + (size_t)m0 * K, (unsigned long long)rows_a * (unsigned long long)K);
+        rsB = make_buffer_resource(B + (size_t)n0 * K, (unsigned long long)rows_b * (unsigned long long)K);
         kt_base = kt0;
         kt_count = count;
         const unsigned key = rotate == 1 ? (unsigned)tile_n : (unsigned)item;   // item: (round, XCD)
@@ -199,17 +210,29 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         kt_rot = rotate == 0 ? 0 : __builtin_amdgcn_readfirstlane((int)(((key * 2654435761u) >> 8) % (unsigned)count));
     };
     // load number j (0 .. LOADS-1) of step `ktile` of the planned item's K walk into ring slot `stage`
-    auto issue_load = [&](int j, int ktile, int stage) {
+    // (the lambdas around the loads are forced inline: a closure left in memory would turn the
+    // scalar operands of the load instruction into per-lane values)
+    auto issue_load = [&](int j, int ktile, int stage) __attribute__((always_inline)) {
         int kk = ktile + kt_rot;
         kk = kk >= kt_count ? kk - kt_count : kk;
-        const uint32_t koff = (uint32_t)((kt_base + kk) * BK);
+        // (pinned to a scalar register: it is an SGPR operand of the load and also feeds per-lane arithmetic)
+        const uint32_t koff = (uint32_t)__builtin_amdgcn_readfirstlane((kt_base + kk) * BK);
         const uint32_t sbase = (uint32_t)(stage * S::STAGE_BYTES);
+        // the K tile that overhangs K: chunks past the end of the row go outside the extent
+        uint32_t voff = ld_off[j];
+        if (KOVER && kt_base + kk == KT - 1) {                      // uniform, rarely taken
+            const int jj = j < S::A_LOADS ? j : j - S::A_LOADS;
+            const int per = j < S::A_LOADS ? S::A_LOADS : S::B_LOADS;
+            const int row = (wave * per + jj) * RPI + lrow;
+            const uint32_t kpos = koff + (uint32_t)((lslot ^ tile_swizzle<BK, S::SWZ>(row)) * 16);
+            voff = kpos >= (uint32_t)K ? 0xFFFFFFF0u : voff;
+        }
         if (j < S::A_LOADS)
-            buffer_load_lds_b128(rsA, ldsA + sbase + (uint32_t)(j * RPI * BK), ld_off[j], koff);
+            buffer_load_lds_b128(rsA, ldsA + sbase + (uint32_t)(j * RPI * BK), voff, koff);
         else
-            buffer_load_lds_b128(rsB, ldsB + sbase + (uint32_t)((j - S::A_LOADS) * RPI * BK), ld_off[j], koff);
+            buffer_load_lds_b128(rsB, ldsB + sbase + (uint32_t)((j - S::A_LOADS) * RPI * BK), voff, koff);
     };
-    auto issue_all_loads = [&](int ktile, int stage) {
+    auto issue_all_loads = [&](int ktile, int stage) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < S::LOADS; ++j) issue_load(j, ktile, stage);
     };

@@ -53,7 +53,8 @@ def test_kernel_selection_is_pure_host_logic(pkg):
     assert L.fp8gemm_select_algo(1, 28672, 8192) == pkg.ALGO_SKINNY
     assert L.fp8gemm_select_algo(64, 8192, 10240) == pkg.ALGO_SKINNY
     assert L.fp8gemm_select_algo(256, 8192, 28672) == pkg.ALGO_TILE
-    assert L.fp8gemm_select_algo(100, 100, 100) == pkg.ALGO_DIRECT       # k not a multiple of 64
+    assert L.fp8gemm_select_algo(100, 100, 100) == pkg.ALGO_DIRECT       # k not a multiple of 16
+    assert L.fp8gemm_select_algo(100, 112, 100) == pkg.ALGO_TILE         # k a multiple of 16: the last K tile overhangs
     assert L.fp8gemm_select_algo(512, 192, 512) == pkg.ALGO_TILE         # odd count of 64-byte K tiles
     assert L.fp8gemm_select_algo(16, 100, 64) == pkg.ALGO_DIRECT
     assert L.fp8gemm_select_algo(0, 1, 1) == -1

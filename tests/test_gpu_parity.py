@@ -156,6 +156,26 @@ def test_tile_k_slices_for_the_last_partial_round(pkg, oracle, variant, split, s
     assert np.isfinite(C).all()
 
 
+@pytest.mark.parametrize("variant", [None, 0, 1, 5, 6])
+@pytest.mark.parametrize("shape", [(256, 16, 256), (300, 1000 // 16 * 16 + 16, 200), (512, 2000, 520), (1100, 4112, 700),
+                                   (64, 1040, 512), (16, 8176, 1024)])
+def test_k_that_is_only_a_multiple_of_16(pkg, oracle, variant, shape):
+    """The last K tile overhangs K: its bytes past the end of each row must count as zeros,
+    not as the next row's bytes.  Every persistent tile shape, and the automatic selection
+    (which no longer needs the general kernel for these)."""
+    M, K, N = shape
+    assert K % 16 == 0 and K % 64 != 0
+    assert pkg.lib().fp8gemm_select_algo(M, K, N) == ALGOS["tile"]
+    A = pkg.fill((M, K), 1, seed=0xA11CE + K, dist="normal", sigma=4.0)
+    B = pkg.fill((N, K), 0, seed=0xB0B + K, dist="normal", sigma=4.0)
+    if variant is None:
+        C = run_gpu(pkg, A, 1, B, 0)
+    else:
+        C = run_gpu(pkg, A, 1, B, 0, algo=ALGOS["tile"], variant=variant)
+    worst = assert_within_bound(oracle, C, A, 1, B, 0, hw_term=K < 1024)
+    assert worst < 0.5
+
+
 @pytest.mark.parametrize("variant", [1, 7, None])
 @pytest.mark.parametrize("shape", [(256, 64, 256), (300, 192, 200), (1100, 448, 2100), (2048, 8256, 2304)])
 def test_odd_count_of_64_byte_k_tiles(pkg, oracle, variant, shape):
