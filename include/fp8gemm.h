@@ -62,6 +62,24 @@ int fp8gemm_e5m2_e4m3_stage4(int m, int k, int n, const void *a, const void *b, 
 int fp8gemm_launch(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
                    float *out, int stages, void *stream);
 
+/*
+ * Extended epilogue, with no counterpart in the reference's gemm:: API; it covers what the
+ * reference's vendor-library sample passes to cuBLASLt next to the operands (host alpha,
+ * device pointers to per-tensor scales of A and B: GEMM/src/cublas.cu:9-16, 41-42) and a
+ * 16-bit output:
+ *     out[i*n+j] = cast_out_type( alpha * a_scale * b_scale * sum_t a[i*k+t] * b[j*k+t] )
+ * with the sum accumulated in fp32 as in fp8gemm_launch, the scaling done in fp32 and one
+ * rounding to nearest even at the end.  out_type: FP8GEMM_OUT_F32 (float), FP8GEMM_OUT_BF16,
+ * FP8GEMM_OUT_F16 (2-byte elements).  a_scale / b_scale: device pointers to one float each,
+ * read by the kernel when it runs, or NULL for 1.  Pure overwrite: out is never read (no beta).
+ */
+#define FP8GEMM_OUT_F32 0
+#define FP8GEMM_OUT_BF16 1
+#define FP8GEMM_OUT_F16 2
+int fp8gemm_launch_ex(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
+                      void *out, int out_type, float alpha, const float *a_scale, const float *b_scale,
+                      void *stream);
+
 /* As fp8gemm_launch, but forces one kernel family (FP8GEMM_ALGO_*).  Returns
  * hipErrorInvalidValue when the family cannot run the shape. */
 int fp8gemm_launch_algo(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,

@@ -66,6 +66,8 @@ def lib():
         fn.argtypes = [ci, ci, ci, vp, vp, vp]
     L.fp8gemm_launch.restype = ci
     L.fp8gemm_launch.argtypes = [ci, ci, ci, vp, ci, vp, ci, vp, ci, vp]
+    L.fp8gemm_launch_ex.restype = ci
+    L.fp8gemm_launch_ex.argtypes = [ci, ci, ci, vp, ci, vp, ci, vp, ci, ctypes.c_float, vp, vp, vp]
     L.fp8gemm_launch_algo.restype = ci
     L.fp8gemm_launch_algo.argtypes = [ci, ci, ci, vp, ci, vp, ci, vp, ci, ci, vp]
     L.fp8gemm_launch_tuned.restype = ci
@@ -197,6 +199,34 @@ def gemm(a, b, out=None, a_fmt=None, b_fmt=None, stages=2, algo=ALGO_AUTO, varia
         code = L.fp8gemm_launch_tuned(m, k, n, a.data_ptr(), fa, b.data_ptr(), fb, out.data_ptr(), algo,
                                       -1 if variant is None else variant, split_k, s)
     check(code)
+    return out
+
+
+OUT_F32, OUT_BF16, OUT_F16 = 0, 1, 2
+
+
+def gemm_ex(a, b, out_dtype=None, out=None, alpha=1.0, a_scale=None, b_scale=None, a_fmt=None, b_fmt=None,
+            stream=None):
+    """out[m, n] = cast(alpha * a_scale * b_scale * sum_k a[m, k] * b[n, k]) through
+    fp8gemm_launch_ex.  out_dtype: torch.float32 / bfloat16 / float16; a_scale, b_scale:
+    one-element float32 device tensors or None."""
+    import torch
+    if not (a.is_cuda and b.is_cuda and a.is_contiguous() and b.is_contiguous()):
+        raise Fp8GemmError("operands must be contiguous device tensors")
+    m, k = a.shape
+    n, k2 = b.shape
+    if k != k2:
+        raise Fp8GemmError("inner dimensions differ: %d vs %d" % (k, k2))
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype or torch.float32, device=a.device)
+    code = {torch.float32: OUT_F32, torch.bfloat16: OUT_BF16, torch.float16: OUT_F16}[out.dtype]
+    for s in (a_scale, b_scale):
+        if s is not None and not (s.is_cuda and s.dtype == torch.float32 and s.numel() == 1):
+            raise Fp8GemmError("scales are one-element float32 device tensors")
+    check(lib().fp8gemm_launch_ex(m, k, n, a.data_ptr(), _fmt_of(a, a_fmt), b.data_ptr(), _fmt_of(b, b_fmt),
+                                  out.data_ptr(), code, float(alpha),
+                                  None if a_scale is None else a_scale.data_ptr(),
+                                  None if b_scale is None else b_scale.data_ptr(), _stream_handle(stream)))
     return out
 
 

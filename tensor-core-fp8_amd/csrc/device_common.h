@@ -44,4 +44,59 @@ __device__ __forceinline__ v8i pack8(v4i lo, v4i hi)
     return r;
 }
 
+// What a kernel does with a finished fp32 sum: multiply by alpha * a_scale * b_scale and
+// store as fp32, bf16 or fp16 (round to nearest even).  The scale pointers are device
+// pointers to one float each, or null for 1.  The plain entry points use {1, null, null,
+// fp32}: the multiplication by 1.0f is exact, results are the bare sums.
+#define FP8GEMM_DEV_OUT_F32 0
+#define FP8GEMM_DEV_OUT_BF16 1
+#define FP8GEMM_DEV_OUT_F16 2
+struct OutSpec {
+    float alpha;
+    const float *a_scale;
+    const float *b_scale;
+    int type;
+};
+
+__device__ __forceinline__ float out_scale(const OutSpec &o)
+{
+    float s = o.alpha;
+    if (o.a_scale) s *= *o.a_scale;
+    if (o.b_scale) s *= *o.b_scale;
+    return s;
+}
+
+__device__ __forceinline__ uint32_t out_bits16(float v, int type)
+{
+    if (type == FP8GEMM_DEV_OUT_BF16) {
+        const __bf16 h = (__bf16)v;
+        return (uint32_t)__builtin_bit_cast(unsigned short, h);
+    }
+    const _Float16 h = (_Float16)v;
+    return (uint32_t)__builtin_bit_cast(unsigned short, h);
+}
+
+// element `index` of an output matrix of the given type
+__device__ __forceinline__ void store_out(void *base, size_t index, float v, int type)
+{
+    if (type == FP8GEMM_DEV_OUT_F32)
+        static_cast<float *>(base)[index] = v;
+    else
+        static_cast<unsigned short *>(base)[index] = (unsigned short)out_bits16(v, type);
+}
+
+// four consecutive elements starting at `index` (index % 4 == 0, 16-byte aligned base)
+__device__ __forceinline__ void store_out4(void *base, size_t index, v4f v, int type)
+{
+    if (type == FP8GEMM_DEV_OUT_F32) {
+        *reinterpret_cast<v4f *>(static_cast<float *>(base) + index) = v;
+    } else {
+        typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+        v2u w;
+        w[0] = out_bits16(v[0], type) | (out_bits16(v[1], type) << 16);
+        w[1] = out_bits16(v[2], type) | (out_bits16(v[3], type) << 16);
+        *reinterpret_cast<v2u *>(static_cast<unsigned short *>(base) + index) = w;
+    }
+}
+
 #endif  // FP8GEMM_DEVICE_COMMON_H

@@ -107,37 +107,37 @@ hipError_t allow_lds(Kernel kernel, int bytes)
 
 template <class S, int AF, int BF>
 struct TileKernelTag {};
-template <class S, int AF, int BF, bool KOVER>
+template <class S, int AF, int BF, bool KOVER, bool EX>
 struct PtileKernelTag {};
 template <class S, int AF, int BF>
 struct SkinnyKernelTag {};
 
 // out[i] = sum over the nsplit planes of ws, on `stream`
-hipError_t launch_reduce(const float *ws, float *out, size_t count, int nsplit, hipStream_t stream)
+hipError_t launch_reduce(const float *ws, void *out, size_t count, int nsplit, const OutSpec &spec, hipStream_t stream)
 {
     const bool vec = count % 4 == 0 &&
                      ((reinterpret_cast<uintptr_t>(ws) | reinterpret_cast<uintptr_t>(out)) % 16) == 0;
     if (vec) {
         const size_t count4 = count / 4;
         hipLaunchKernelGGL(gemm_splitk_reduce4_kernel, dim3((unsigned)((count4 + 255) / 256)), dim3(256), 0, stream,
-                           reinterpret_cast<const v4f *>(ws), reinterpret_cast<v4f *>(out), count4, nsplit);
+                           reinterpret_cast<const v4f *>(ws), out, count4, nsplit, spec);
     } else {
         hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
-                           ws, out, count, nsplit);
+                           ws, out, count, nsplit, spec);
     }
     return hipGetLastError();
 }
 
 // ------------------------------------------------------------------ direct
 template <int AF, int BF>
-hipError_t launch_direct(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
-                         hipStream_t stream)
+hipError_t launch_direct(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
+                         const OutSpec &spec, hipStream_t stream)
 {
     const long gy = (m + 31) / 32, gx = (n + 31) / 32;
     if (gy > 65535) return hipErrorInvalidValue;
     const bool vec_ok = (k % 16 == 0) && ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) % 16 == 0);
     hipLaunchKernelGGL((gemm_direct_kernel<AF, BF>), dim3((unsigned)gx, (unsigned)gy), dim3(64), 0, stream,
-                       m, k, n, a, b, out, vec_ok ? 1 : 0);
+                       m, k, n, a, b, out, vec_ok ? 1 : 0, spec);
     return hipGetLastError();
 }
 
@@ -198,9 +198,9 @@ size_t ptile_scratch_bytes(const PtileWork &w, int bm, int bn)
 
 // persistent form: one workgroup per CU walks its share of the work list; the K slices'
 // partial sums go through the scratch buffer and a reduction pass
-template <class S, int AF, int BF, bool KOVER>
-hipError_t launch_ptile_shape_k(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
-                                int nsplit, bool split_all, int rotate, hipStream_t stream)
+template <class S, int AF, int BF, bool KOVER, bool EX>
+hipError_t launch_ptile_shape_k(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
+                                int nsplit, bool split_all, int rotate, const OutSpec &spec, hipStream_t stream)
 {
     if (k % 16 != 0 || k > (1 << 23) || nsplit < 1 || nsplit > (k + S::BK - 1) / S::BK) return hipErrorInvalidValue;
     const PtileWork w = ptile_work(m, n, S::BM, S::BN, nsplit, split_all);
@@ -212,49 +212,66 @@ hipError_t launch_ptile_shape_k(int m, int k, int n, const uint8_t *a, const uin
         if (e != hipSuccess) return e;
         ws = static_cast<float *>(p);
     }
-    auto kernel = gemm_ptile_kernel<S, AF, BF, KOVER>;
-    hipError_t e = allow_lds<PtileKernelTag<S, AF, BF, KOVER>>(kernel, S::PTILE_LDS_BYTES);
+    auto kernel = gemm_ptile_kernel<S, AF, BF, KOVER, EX>;
+    hipError_t e = allow_lds<PtileKernelTag<S, AF, BF, KOVER, EX>>(kernel, S::PTILE_LDS_BYTES);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * w.slots)), dim3(S::THREADS), S::PTILE_LDS_BYTES, stream,
-                       m, k, n, a, b, out, ws, w.tiles_m, w.tiles_n, w.GM, w.bulk, w.tail, w.nsplit, w.rounds, rotate);
+                       m, k, n, a, b, out, ws, w.tiles_m, w.tiles_n, w.GM, w.bulk, w.tail, w.nsplit, w.rounds, rotate, spec);
     e = hipGetLastError();
     if (e != hipSuccess || w.nsplit == 1) return e;
     const size_t threads = (size_t)w.tail * (S::BM * S::BN / 4);
     hipLaunchKernelGGL(gemm_tile_slices_reduce_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream,
-                       ws, out, m, n, S::BM, S::BN, w.tiles_m, w.tiles_n, w.GM, w.bulk, w.tail, w.nsplit);
+                       ws, out, m, n, S::BM, S::BN, w.tiles_m, w.tiles_n, w.GM, w.bulk, w.tail, w.nsplit, spec);
     return hipGetLastError();
 }
 
-// OVERHANG_TOO: this shape is also compiled for a K that is not a multiple of its K tile
-template <class S, int AF, int BF, bool OVERHANG_TOO>
-hipError_t launch_ptile_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
-                              int nsplit, bool split_all, int rotate, hipStream_t stream)
+bool plain_output(const OutSpec &spec)
 {
-    if (k % S::BK == 0)
-        return launch_ptile_shape_k<S, AF, BF, false>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
-    if constexpr (OVERHANG_TOO)
-        return launch_ptile_shape_k<S, AF, BF, true>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
-    else
+    return spec.type == FP8GEMM_DEV_OUT_F32 && spec.alpha == 1.0f && !spec.a_scale && !spec.b_scale;
+}
+
+// OVERHANG_TOO: this shape is also compiled for a K that is not a multiple of its K tile.
+// EX_TOO: ... and for the extended epilogue (scale, 16-bit output).
+template <class S, int AF, int BF, bool OVERHANG_TOO, bool EX_TOO>
+hipError_t launch_ptile_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
+                              int nsplit, bool split_all, int rotate, const OutSpec &spec, hipStream_t stream)
+{
+    const bool over = k % S::BK != 0;
+    if (plain_output(spec)) {
+        if (!over)
+            return launch_ptile_shape_k<S, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+        if constexpr (OVERHANG_TOO)
+            return launch_ptile_shape_k<S, AF, BF, true, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
         return hipErrorInvalidValue;
+    }
+    if constexpr (EX_TOO) {
+        if (!over)
+            return launch_ptile_shape_k<S, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+        if constexpr (OVERHANG_TOO)
+            return launch_ptile_shape_k<S, AF, BF, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+    }
+    return hipErrorInvalidValue;
 }
 
 template <int AF, int BF>
-hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
-                       int variant, int nsplit, bool split_all, int rotate, hipStream_t stream)
+hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
+                       int variant, int nsplit, bool split_all, int rotate, const OutSpec &spec, hipStream_t stream)
 {
     const bool persistent = !(variant == 3 || variant == 4 || variant == 7);
     if (!persistent && nsplit != 1) return hipErrorInvalidValue;   // K slices only in the persistent kernels
+    // the one-tile-per-workgroup kernels write bare fp32 sums only
+    if (!persistent && !plain_output(spec)) return hipErrorInvalidValue;
     switch (variant) {
-    case 0: return launch_ptile_shape<TileP2, AF, BF, true>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
-    case 1: return launch_ptile_shape<TileP4, AF, BF, true>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
-    case 2: return launch_ptile_shape<TileP8, AF, BF, false>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
-    case 3: return launch_tile_shape<TileS2, AF, BF>(m, k, n, a, b, out, stream);
-    case 4: return launch_tile_shape<TileS4, AF, BF>(m, k, n, a, b, out, stream);
-    case 5: return launch_ptile_shape<TileH3, AF, BF, true>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
-    case 6: return launch_ptile_shape<TileQ2, AF, BF, true>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
-    case 7: return launch_tile_shape<TileS64, AF, BF>(m, k, n, a, b, out, stream);
-    case 8: return launch_ptile_shape<TileW3, AF, BF, false>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
-    case 9: return launch_ptile_shape<TileT2, AF, BF, false>(m, k, n, a, b, out, nsplit, split_all, rotate, stream);
+    case 0: return launch_ptile_shape<TileP2, AF, BF, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+    case 1: return launch_ptile_shape<TileP4, AF, BF, true, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+    case 2: return launch_ptile_shape<TileP8, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+    case 3: return launch_tile_shape<TileS2, AF, BF>(m, k, n, a, b, static_cast<float *>(out), stream);
+    case 4: return launch_tile_shape<TileS4, AF, BF>(m, k, n, a, b, static_cast<float *>(out), stream);
+    case 5: return launch_ptile_shape<TileH3, AF, BF, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+    case 6: return launch_ptile_shape<TileQ2, AF, BF, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+    case 7: return launch_tile_shape<TileS64, AF, BF>(m, k, n, a, b, static_cast<float *>(out), stream);
+    case 8: return launch_ptile_shape<TileW3, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+    case 9: return launch_ptile_shape<TileT2, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -265,36 +282,36 @@ struct SkinnyPlan {
 };
 
 template <class S, int AF, int BF>
-hipError_t launch_skinny_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
-                               int nsplit, hipStream_t stream)
+hipError_t launch_skinny_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
+                               int nsplit, const OutSpec &spec, hipStream_t stream)
 {
     if (m > S::MP || n % S::NP != 0 || nsplit < 1 || k % nsplit != 0 || (k / nsplit) % S::BK != 0)
         return hipErrorInvalidValue;
     const int ngroups = n / S::NP;
     const int kchunk = k / nsplit;
-    float *dst = out;
+    void *dst = out;
     if (nsplit > 1) {
         void *ws = nullptr;
         hipError_t e = scratch_get((size_t)nsplit * m * n * sizeof(float), &ws);
         if (e != hipSuccess) return e;
-        dst = static_cast<float *>(ws);
+        dst = ws;
     }
     auto kernel = gemm_skinny_kernel<S, AF, BF>;
     hipError_t e = allow_lds<SkinnyKernelTag<S, AF, BF>>(kernel, S::LDS_BYTES);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3((unsigned)(ngroups * nsplit)), dim3(64), S::LDS_BYTES, stream,
-                       m, k, n, a, b, dst, ngroups, kchunk);
+                       m, k, n, a, b, dst, ngroups, kchunk, nsplit, spec);
     e = hipGetLastError();
     if (e != hipSuccess || nsplit == 1) return e;
-    return launch_reduce(dst, out, (size_t)m * n, nsplit, stream);
+    return launch_reduce(static_cast<const float *>(dst), out, (size_t)m * n, nsplit, spec, stream);
 }
 
 template <template <int, int> class V, int AF, int BF>
-hipError_t launch_skinny_mt(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
-                            const SkinnyPlan &p, hipStream_t stream)
+hipError_t launch_skinny_mt(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
+                            const SkinnyPlan &p, const OutSpec &spec, hipStream_t stream)
 {
 #define SK(MT, TN) \
-    if (p.mt == MT && p.tn == TN) return launch_skinny_shape<V<MT, TN>, AF, BF>(m, k, n, a, b, out, p.nsplit, stream);
+    if (p.mt == MT && p.tn == TN) return launch_skinny_shape<V<MT, TN>, AF, BF>(m, k, n, a, b, out, p.nsplit, spec, stream);
     SK(1, 1) SK(1, 2) SK(1, 4)
     SK(2, 1) SK(2, 2) SK(2, 4)
     SK(3, 1) SK(3, 2) SK(3, 4)
@@ -304,16 +321,16 @@ hipError_t launch_skinny_mt(int m, int k, int n, const uint8_t *a, const uint8_t
 }
 
 template <int AF, int BF>
-hipError_t launch_skinny(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
-                         const SkinnyPlan &p, hipStream_t stream)
+hipError_t launch_skinny(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
+                         const SkinnyPlan &p, const OutSpec &spec, hipStream_t stream)
 {
     switch (p.variant) {
-    case 0: return launch_skinny_mt<SkinnyV0, AF, BF>(m, k, n, a, b, out, p, stream);
-    case 1: return launch_skinny_mt<SkinnyV1, AF, BF>(m, k, n, a, b, out, p, stream);
-    case 2: return launch_skinny_mt<SkinnyV2, AF, BF>(m, k, n, a, b, out, p, stream);
-    case 3: return launch_skinny_mt<SkinnyV3, AF, BF>(m, k, n, a, b, out, p, stream);
-    case 4: return launch_skinny_mt<SkinnyV4, AF, BF>(m, k, n, a, b, out, p, stream);
-    case 5: return launch_skinny_mt<SkinnyV5, AF, BF>(m, k, n, a, b, out, p, stream);
+    case 0: return launch_skinny_mt<SkinnyV0, AF, BF>(m, k, n, a, b, out, p, spec, stream);
+    case 1: return launch_skinny_mt<SkinnyV1, AF, BF>(m, k, n, a, b, out, p, spec, stream);
+    case 2: return launch_skinny_mt<SkinnyV2, AF, BF>(m, k, n, a, b, out, p, spec, stream);
+    case 3: return launch_skinny_mt<SkinnyV3, AF, BF>(m, k, n, a, b, out, p, spec, stream);
+    case 4: return launch_skinny_mt<SkinnyV4, AF, BF>(m, k, n, a, b, out, p, spec, stream);
+    case 5: return launch_skinny_mt<SkinnyV5, AF, BF>(m, k, n, a, b, out, p, spec, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -458,8 +475,8 @@ size_t tile_plan_scratch_bytes(int m, int n, const TilePlan &p)
 }
 
 template <int AF, int BF>
-hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out, int stages,
-                    int algo, int variant, int nsplit, hipStream_t stream)
+hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out, int stages,
+                    int algo, int variant, int nsplit, const OutSpec &spec, hipStream_t stream)
 {
     const bool aligned = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) % 16) == 0;
     if (algo == FP8GEMM_ALGO_AUTO) {
@@ -468,7 +485,7 @@ hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, flo
     }
     switch (algo) {
     case FP8GEMM_ALGO_DIRECT:
-        return launch_direct<AF, BF>(m, k, n, a, b, out, stream);
+        return launch_direct<AF, BF>(m, k, n, a, b, out, spec, stream);
     case FP8GEMM_ALGO_TILE: {
         if (!aligned || k % 16 != 0 || k > (1 << 23)) return hipErrorInvalidValue;
         TilePlan p = plan_tile(m, k, n, stages);
@@ -490,7 +507,7 @@ hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, flo
             p.nsplit = -nsplit;
             p.split_all = false;
         }
-        return launch_tile<AF, BF>(m, k, n, a, b, out, p.variant, p.nsplit, p.split_all, p.rotate, stream);
+        return launch_tile<AF, BF>(m, k, n, a, b, out, p.variant, p.nsplit, p.split_all, p.rotate, spec, stream);
     }
     case FP8GEMM_ALGO_SKINNY: {
         if (!aligned || !skinny_ok(m, k, n)) return hipErrorInvalidValue;
@@ -502,15 +519,17 @@ hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, flo
         }
         if (nsplit > 0) p.nsplit = nsplit;
         if (nsplit < 0) return hipErrorInvalidValue;
-        return launch_skinny<AF, BF>(m, k, n, a, b, out, p, stream);
+        return launch_skinny<AF, BF>(m, k, n, a, b, out, p, spec, stream);
     }
     default:
         return hipErrorInvalidValue;
     }
 }
 
-int launch_checked(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt, float *out,
-                   int stages, int algo, int variant, int nsplit, void *stream)
+const OutSpec kPlainOut = {1.0f, nullptr, nullptr, FP8GEMM_DEV_OUT_F32};
+
+int launch_checked(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt, void *out,
+                   int stages, int algo, int variant, int nsplit, void *stream, const OutSpec &spec = kPlainOut)
 {
     if (m <= 0 || k <= 0 || n <= 0 || !a || !b || !out) return (int)hipErrorInvalidValue;
     if ((a_fmt != FP8GEMM_E4M3 && a_fmt != FP8GEMM_E5M2) || (b_fmt != FP8GEMM_E4M3 && b_fmt != FP8GEMM_E5M2))
@@ -525,13 +544,13 @@ int launch_checked(int m, int k, int n, const void *a, int a_fmt, const void *b,
     (void)hipGetLastError();
     hipError_t e;
     if (a_fmt == FP8GEMM_E4M3 && b_fmt == FP8GEMM_E4M3)
-        e = dispatch<0, 0>(m, k, n, pa, pb, out, stages, algo, variant, nsplit, s);
+        e = dispatch<0, 0>(m, k, n, pa, pb, out, stages, algo, variant, nsplit, spec, s);
     else if (a_fmt == FP8GEMM_E5M2 && b_fmt == FP8GEMM_E5M2)
-        e = dispatch<1, 1>(m, k, n, pa, pb, out, stages, algo, variant, nsplit, s);
+        e = dispatch<1, 1>(m, k, n, pa, pb, out, stages, algo, variant, nsplit, spec, s);
     else if (a_fmt == FP8GEMM_E4M3)
-        e = dispatch<0, 1>(m, k, n, pa, pb, out, stages, algo, variant, nsplit, s);
+        e = dispatch<0, 1>(m, k, n, pa, pb, out, stages, algo, variant, nsplit, spec, s);
     else
-        e = dispatch<1, 0>(m, k, n, pa, pb, out, stages, algo, variant, nsplit, s);
+        e = dispatch<1, 0>(m, k, n, pa, pb, out, stages, algo, variant, nsplit, spec, s);
     return (int)e;
 }
 
@@ -555,6 +574,17 @@ int fp8gemm_launch_tuned(int m, int k, int n, const void *a, int a_fmt, const vo
                          float *out, int algo, int variant, int split_k, void *stream)
 {
     return launch_checked(m, k, n, a, a_fmt, b, b_fmt, out, 2, algo, variant, split_k, stream);
+}
+
+int fp8gemm_launch_ex(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
+                      void *out, int out_type, float alpha, const float *a_scale, const float *b_scale,
+                      void *stream)
+{
+    if (out_type != FP8GEMM_OUT_F32 && out_type != FP8GEMM_OUT_BF16 && out_type != FP8GEMM_OUT_F16)
+        return (int)hipErrorInvalidValue;
+    if (!(alpha == alpha)) return (int)hipErrorInvalidValue;      // NaN
+    const OutSpec spec = {alpha, a_scale, b_scale, out_type};
+    return launch_checked(m, k, n, a, a_fmt, b, b_fmt, out, 2, FP8GEMM_ALGO_AUTO, -1, 0, stream, spec);
 }
 
 int fp8gemm_num_variants(int algo)

@@ -36,7 +36,7 @@ template <int AF, int BF>
 __global__ __launch_bounds__(64) void gemm_direct_kernel(int M, int K, int N,
                                                          const uint8_t *__restrict__ A,
                                                          const uint8_t *__restrict__ B,
-                                                         float *__restrict__ C, int vec_ok)
+                                                         void *__restrict__ C, int vec_ok, OutSpec spec)
 {
     const int lane = threadIdx.x;
     const int i = lane & 31;
@@ -55,9 +55,10 @@ __global__ __launch_bounds__(64) void gemm_direct_kernel(int M, int K, int N,
 
     const int col = n0 + i;
     if (col < N) {
+        const float scale = out_scale(spec);
         for (int r = 0; r < 16; ++r) {
             const int row = m0 + 8 * (r >> 2) + 4 * g + (r & 3);
-            if (row < M) C[(size_t)row * N + col] = acc[r];
+            if (row < M) store_out(C, (size_t)row * N + col, acc[r] * scale, spec.type);
         }
     }
 }

@@ -75,16 +75,17 @@ __device__ __forceinline__ v4i make_buffer_resource(const void *base, unsigned l
 }
 
 // KOVER: the last K tile may overhang K (K % BK != 0); compiled separately so that the
-// common case carries no test for it.
-template <class S, int AF, int BF, bool KOVER>
+// common case carries no test for it.  EX: the output goes through `spec` (scale, fp32 /
+// bf16 / fp16); without it C receives the bare fp32 sums and `spec` is ignored.
+template <class S, int AF, int BF, bool KOVER, bool EX>
 __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, int N,
                                                                  const uint8_t *__restrict__ A,
                                                                  const uint8_t *__restrict__ B,
-                                                                 float *__restrict__ C,
+                                                                 void *__restrict__ C,
                                                                  float *__restrict__ ws,
                                                                  int tiles_m, int tiles_n, int GM,
                                                                  int bulk, int tail, int nsplit,
-                                                                 int rounds, int rotate)
+                                                                 int rounds, int rotate, OutSpec spec)
 {
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, CH = S::CH, RPI = S::RPI;
     constexpr int STAGES = S::STAGES, TM = S::TM, TN = S::TN, KSTEPS = S::KSTEPS;
@@ -389,17 +390,21 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         const int wcol0 = n0 + wn * (BN / S::WN);
         // destination of this item: its tile of C (row stride N), or a whole BM x BN slot of
         // the scratch (row stride BN; rows and columns past the matrix hold zeros)
+        // (the scratch takes bare fp32 sums; scale and output type are applied where C is written)
         const bool to_ws = ws_slot >= 0;
-        float *__restrict__ tile_out = to_ws ? ws + (size_t)ws_slot * (size_t)(BM * BN)
-                                             : C + (size_t)m0 * (size_t)N + n0;
+        void *__restrict__ tile_base = to_ws ? static_cast<void *>(ws) : C;
+        const size_t tile_origin = to_ws ? (size_t)ws_slot * (size_t)(BM * BN) : (size_t)m0 * (size_t)N + n0;
         const size_t ldo = to_ws ? (size_t)BN : (size_t)N;
+        const int otype = (!EX || to_ws) ? FP8GEMM_DEV_OUT_F32 : spec.type;
+        const float oscale = (!EX || to_ws) ? 1.0f : out_scale(spec);
         const bool full = to_ws || ((m0 + BM <= M) && (n0 + BN <= N) && (N % 4 == 0) &&
                                     (reinterpret_cast<uintptr_t>(C) % 16 == 0));
-        if (full) {
+        {
             // Each wave transposes its results through a private strip of LDS (the part of
             // the ring the next tile's first loads do not use, plus the LDS above the ring)
             // so that every store instruction writes whole contiguous row segments of C:
             // a CU drains full-line stores about three times faster than 32-byte pieces.
+            // Tiles that overhang C take the same route with every element store guarded.
             constexpr int EP = S::EP_COLS;                       // columns staged at a time
             constexpr int ROWB = EP * 4 + 16;                    // padded row: conflict-free both ways
             constexpr int LPR = EP / 4;                          // lanes per row when reading back
@@ -418,27 +423,37 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                             v4f v = {acc[i][j][4 * q4], acc[i][j][4 * q4 + 1], acc[i][j][4 * q4 + 2], acc[i][j][4 * q4 + 3]};
                             lds_store_b128_acc(stg_addr + (uint32_t)(fi * ROWB + (j * 32 - c0 + 8 * q4 + 4 * fg) * 4), v);
                         }
+                    if (!EX && full) {
 #pragma unroll
-                    for (int r0 = 0; r0 < 32; r0 += RPI_ST) {
-                        const v4f v = *reinterpret_cast<const v4f *>(stg + (r0 + rl) * ROWB + cl * 16);
-                        float *dst = tile_out + (size_t)(wrow0 - m0 + i * 32 + r0 + rl) * ldo + (wcol0 - n0 + c0 + cl * 4);
-                        *reinterpret_cast<v4f *>(dst) = v;
+                        for (int r0 = 0; r0 < 32; r0 += RPI_ST) {
+                            const v4f v = *reinterpret_cast<const v4f *>(stg + (r0 + rl) * ROWB + cl * 16);
+                            store_out4(tile_base, tile_origin + (size_t)(wrow0 - m0 + i * 32 + r0 + rl) * ldo + (wcol0 - n0 + c0 + cl * 4),
+                                       v, FP8GEMM_DEV_OUT_F32);
+                        }
+                    } else {
+                        // scale and convert (EX), guard (tiles that overhang C); a few rows at a time
+#pragma unroll 2
+                        for (int r0 = 0; r0 < 32; r0 += RPI_ST) {
+                            v4f v = *reinterpret_cast<const v4f *>(stg + (r0 + rl) * ROWB + cl * 16);
+                            if (EX) {
+                                v[0] *= oscale;
+                                v[1] *= oscale;
+                                v[2] *= oscale;
+                                v[3] *= oscale;
+                            }
+                            const int lrow_ = wrow0 - m0 + i * 32 + r0 + rl;       // inside the tile
+                            const int lcol_ = wcol0 - n0 + c0 + cl * 4;
+                            const size_t index = tile_origin + (size_t)lrow_ * ldo + lcol_;
+                            if (full) {
+                                store_out4(tile_base, index, v, otype);
+                            } else if (m0 + lrow_ < M) {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e)
+                                    if (n0 + lcol_ + e < N) store_out(tile_base, index + e, v[e], otype);
+                            }
+                        }
                     }
                 }
-        } else {
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const int row = wrow0 + i * 32 + fi;
-                if (row < M) {
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-#pragma unroll
-                        for (int q = 0; q < 16; ++q) {
-                            const int col = wcol0 + j * 32 + 8 * (q >> 2) + 4 * fg + (q & 3);
-                            if (col < N) C[(size_t)row * N + col] = acc[i][j][q];
-                        }
-                }
-            }
         }
         tile_m = next_m;
         tile_n = next_n;

@@ -8,20 +8,20 @@
 #include "device_common.h"
 
 __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float *__restrict__ ws,
-                                                                 float *__restrict__ C,
-                                                                 size_t count, int nsplit)
+                                                                 void *__restrict__ C,
+                                                                 size_t count, int nsplit, OutSpec spec)
 {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= count) return;
     float s = ws[i];
     for (int p = 1; p < nsplit; ++p) s += ws[(size_t)p * count + i];
-    C[i] = s;
+    store_out(C, i, s * out_scale(spec), spec.type);
 }
 
 // count4 = count / 4; requires count % 4 == 0 and 16-byte aligned ws and C
 __global__ __launch_bounds__(256) void gemm_splitk_reduce4_kernel(const v4f *__restrict__ ws,
-                                                                  v4f *__restrict__ C,
-                                                                  size_t count4, int nsplit)
+                                                                  void *__restrict__ C,
+                                                                  size_t count4, int nsplit, OutSpec spec)
 {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= count4) return;
@@ -33,7 +33,12 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce4_kernel(const v4f *__r
         s[2] += v[2];
         s[3] += v[3];
     }
-    C[i] = s;
+    const float scale = out_scale(spec);
+    s[0] *= scale;
+    s[1] *= scale;
+    s[2] *= scale;
+    s[3] *= scale;
+    store_out4(C, i * 4, s, spec.type);
 }
 
 // Partial sums of the persistent tiled kernel: scratch slot s*tail + u holds slice s of
@@ -41,9 +46,10 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce4_kernel(const v4f *__r
 // of a tile adds the slices in ascending order and writes the part that lies inside C.
 // The tile numbering is the kernel's: strips of GM tile rows, down a column first.
 __global__ __launch_bounds__(256) void gemm_tile_slices_reduce_kernel(const float *__restrict__ ws,
-                                                                      float *__restrict__ C, int M, int N,
+                                                                      void *__restrict__ C, int M, int N,
                                                                       int BM, int BN, int tiles_m, int tiles_n,
-                                                                      int GM, int bulk, int tail, int nsplit)
+                                                                      int GM, int bulk, int tail, int nsplit,
+                                                                      OutSpec spec)
 {
     const int quads_per_tile = BM * BN / 4;
     const size_t id = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -73,12 +79,17 @@ __global__ __launch_bounds__(256) void gemm_tile_slices_reduce_kernel(const floa
         s[2] += v[2];
         s[3] += v[3];
     }
-    float *dst = C + (size_t)grow * N + gcol;
+    const float scale = out_scale(spec);
+    s[0] *= scale;
+    s[1] *= scale;
+    s[2] *= scale;
+    s[3] *= scale;
+    const size_t index = (size_t)grow * N + gcol;
     if (gcol + 3 < N && N % 4 == 0 && reinterpret_cast<uintptr_t>(C) % 16 == 0) {
-        *reinterpret_cast<v4f *>(dst) = s;
+        store_out4(C, index, s, spec.type);
     } else {
         for (int e = 0; e < 4; ++e)
-            if (gcol + e < N) dst[e] = s[e];
+            if (gcol + e < N) store_out(C, index + e, s[e], spec.type);
     }
 }
 

@@ -72,8 +72,8 @@ template <class S, int AF, int BF>
 __global__ __launch_bounds__(64) void gemm_skinny_kernel(int M, int K, int N,
                                                          const uint8_t *__restrict__ A,
                                                          const uint8_t *__restrict__ B,
-                                                         float *__restrict__ out,
-                                                         int ngroups, int kchunk)
+                                                         void *__restrict__ out,
+                                                         int ngroups, int kchunk, int nsplit, OutSpec spec)
 {
     constexpr int BK = S::BK, CH = S::CH, RPI = S::RPI, STAGES = S::STAGES;
     constexpr int MT = S::MT, TN = S::TN, MP = S::MP;
@@ -170,7 +170,12 @@ __global__ __launch_bounds__(64) void gemm_skinny_kernel(int M, int K, int N,
         __builtin_amdgcn_sched_barrier(0);
     }
 
-    float *dst = out + (size_t)split * M * N;
+    // with K slices `out` is the fp32 scratch (plane `split`, bare sums; the reduction
+    // applies scale and output type), otherwise the output matrix itself
+    const bool partial = nsplit > 1;
+    const float scale = partial ? 1.0f : out_scale(spec);
+    const int type = partial ? FP8GEMM_DEV_OUT_F32 : spec.type;
+    const size_t plane = partial ? (size_t)split * M * N : 0;
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
@@ -178,7 +183,7 @@ __global__ __launch_bounds__(64) void gemm_skinny_kernel(int M, int K, int N,
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int row = i * 16 + 4 * fq + r;
-                if (row < M) dst[(size_t)row * N + n0 + j * 16 + fi] = acc[i][j][r];
+                if (row < M) store_out(out, plane + (size_t)row * N + n0 + j * 16 + fi, acc[i][j][r] * scale, type);
             }
 }
 

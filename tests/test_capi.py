@@ -42,6 +42,11 @@ def test_argument_validation_needs_no_gpu(pkg):
     for name in pkg.ENTRY_POINTS:
         assert getattr(L, name)(128, 128, 128, None, None, None) == INVALID
         assert getattr(L, name)(128, 0, 128, ok_ptr, ok_ptr, ok_ptr) == INVALID
+    # extended epilogue: output type code and alpha are checked as well
+    assert L.fp8gemm_launch_ex(128, 128, 128, ok_ptr, 0, ok_ptr, 0, ok_ptr, 3, 1.0, None, None, None) == INVALID
+    assert L.fp8gemm_launch_ex(128, 128, 128, ok_ptr, 0, ok_ptr, 0, ok_ptr, 1, float("nan"), None, None, None) == INVALID
+    assert L.fp8gemm_launch_ex(128, 128, 128, ok_ptr, 0, ok_ptr, 0, None, 1, 1.0, None, None, None) == INVALID
+    assert L.fp8gemm_launch_ex(0, 128, 128, ok_ptr, 0, ok_ptr, 0, ok_ptr, 0, 1.0, None, None, None) == INVALID
     assert b"invalid" in L.fp8gemm_error_string(INVALID).lower()
     assert L.fp8gemm_version() >= 100
 
