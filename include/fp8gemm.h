@@ -117,7 +117,7 @@ int fp8gemm_plan(int m, int k, int n, int stages, int plan[4]);
  * only allocation the library ever makes; it is grown on demand, reused by
  * later calls and shared by all streams of the device, so calls that overlap
  * on one device and both need it must be ordered by the caller. */
-size_t fp8gemm_scratch_bytes(int m, int k, int n);
+size_t fp8gemm_scratch_bytes(int m, int k, int n);   /* for the stage-2 plan; the stage-4 plan cuts K the same way */
 
 /* Text for a return code (hipGetErrorString). */
 const char *fp8gemm_error_string(int code);

@@ -34,7 +34,11 @@ using TileQ2 = TileShape<128, 128, 128, 2, 2, 2, 3>;  // persistent, quarter til
 using TileS64 = TileShape<128, 128, 64, 2, 2, 4, 2>;  // one tile per workgroup, 64-byte K tiles
 using TileW3 = TileShape<256, 128, 128, 2, 2, 3, 3>;  // persistent, half-width tile, 3 x 48 KiB ring
 using TileT2 = TileShape<192, 256, 128, 2, 2, 2, 3>;  // persistent, three-quarter-height tile: other tile counts
-constexpr int kNumTileVariants = 10;              // 0 P2, 1 P4, 2 P8, 3 S2, 4 S4, 5 H3, 6 Q2, 7 S64, 8 W3, 9 T2
+// the 4-deep rings of 64-byte K tiles behind the stage-4 entry points, same tile shapes
+using TileT4 = TileShape<192, 256, 64, 2, 2, 4, 2>;
+using TileH4 = TileShape<128, 256, 64, 2, 2, 4, 2>;
+using TileQ4 = TileShape<128, 128, 64, 2, 2, 4, 2>;
+constexpr int kNumTileVariants = 13;              // 0 P2, 1 P4, 2 P8, 3 S2, 4 S4, 5 H3, 6 Q2, 7 S64, 8 W3, 9 T2, 10 T4, 11 H4, 12 Q4
 
 // Skinny kernel shapes: <MT, TN, BK, stages>.
 template <int MT, int TN>
@@ -272,6 +276,9 @@ hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, 
     case 7: return launch_tile_shape<TileS64, AF, BF>(m, k, n, a, b, static_cast<float *>(out), stream);
     case 8: return launch_ptile_shape<TileW3, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
     case 9: return launch_ptile_shape<TileT2, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+    case 10: return launch_ptile_shape<TileT4, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+    case 11: return launch_ptile_shape<TileH4, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+    case 12: return launch_ptile_shape<TileQ4, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -396,15 +403,15 @@ struct TilePlan {
 //   K slices add one reduction pass over (nsplit + 1) x the cut tiles.
 // The model only has to rank the candidates, not to predict the time.
 struct PtileCost {
-    int variant, bm, bn;
+    int variant, variant4, bm, bn;              // variant4: the same tile with a 4-deep ring of 64-byte K tiles (-1: none)
     double per_k_tile, per_item, stream_rate;   // us, us, bytes per us
 };
 constexpr PtileCost kPtileCosts[] = {
-    {0, 256, 256, 1.40, 13.0, 4.0e6},
-    {9, 192, 256, 1.25, 11.0, 4.6e6},
-    {5, 128, 256, 1.00, 8.0, 5.0e6},
-    {6, 128, 128, 0.75, 4.5, 3.2e6},
-    {8, 256, 128, 0.90, 10.0, 4.0e6},
+    {0, 1, 256, 256, 1.40, 13.0, 4.0e6},
+    {9, 10, 192, 256, 1.25, 11.0, 4.6e6},
+    {5, 11, 128, 256, 1.00, 8.0, 5.0e6},
+    {6, 12, 128, 128, 0.75, 4.5, 3.2e6},
+    {8, -1, 256, 128, 0.90, 10.0, 4.0e6},
 };
 constexpr double kIdleChipFactor = 0.5;
 constexpr int kSplitChoices[] = {1, 2, 3, 4, 6, 8, 12, 16};
@@ -413,21 +420,20 @@ constexpr size_t kMaxSplitScratch = (size_t)1 << 30;
 
 TilePlan plan_tile(int m, int k, int n, int stages)
 {
-    const long tiles256 = (long)((m + 255) / 256) * ((n + 255) / 256);
-    const bool small = tiles256 < 192;
     TilePlan best = {0, 1, 2, false};
-    if (stages == 4) {                  // the 4-deep rings: one shape for big problems, one for small
-        best.variant = (small && k % 128 == 0) ? 4 : 1;       // (the small one needs whole 128-byte K tiles)
-        return best;
-    }
     const int kt = (k + 127) / 128;
     double best_cost = 1e30;
     for (const PtileCost &c : kPtileCosts) {
         // the 256 x 128 tile pays off where it holds all rows of A at once (no second
         // row of tiles re-reading the same B rows) and is at least half full
         if (c.variant == 8 && (m <= 128 || m > 256)) continue;
-        // a K that is not a multiple of 128: only the shapes compiled for an overhanging K tile
-        if (k % 128 != 0 && !(c.variant == 0 || c.variant == 5 || c.variant == 6)) continue;
+        if (stages == 4) {
+            // the 4-deep rings rank like their 2- and 3-deep twins (same tiles, same work list);
+            // only the 256 x 256 one is compiled for a K that is not a multiple of its K tile
+            if (c.variant4 < 0 || (k % 64 != 0 && c.variant4 != 1)) continue;
+        } else if (k % 128 != 0 && !(c.variant == 0 || c.variant == 5 || c.variant == 6)) {
+            continue;      // overhanging K tile: only the shapes compiled for it
+        }
         for (int mode = 0; mode < 2; ++mode)          // 0: slices for the tail tiles only, 1: for all
             for (int split : kSplitChoices) {
                 if (mode == 1 && split == 1) continue;      // same as mode 0
@@ -451,7 +457,7 @@ TilePlan plan_tile(int m, int k, int n, int stages)
                 if (w.nsplit > 1) cost += 4.0 + (w.nsplit + 1) * (double)w.tail * c.bm * c.bn * 4.0 / 6.0e6;
                 if (cost < best_cost) {
                     best_cost = cost;
-                    best.variant = c.variant;
+                    best.variant = stages == 4 ? c.variant4 : c.variant;
                     best.nsplit = w.nsplit;
                     best.split_all = mode == 1;
                 }
@@ -467,7 +473,7 @@ size_t tile_plan_scratch_bytes(int m, int n, const TilePlan &p)
 {
     if (p.nsplit <= 1) return 0;
     for (const PtileCost &c : kPtileCosts)
-        if (c.variant == p.variant) {
+        if (c.variant == p.variant || c.variant4 == p.variant) {
             const PtileWork w = ptile_work(m, n, c.bm, c.bn, p.nsplit, p.split_all);
             return w.ok ? ptile_scratch_bytes(w, c.bm, c.bn) : 0;
         }

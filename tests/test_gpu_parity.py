@@ -107,7 +107,7 @@ def test_normal_inputs_within_fp32_reordering_bound(pkg, oracle, fa, fb, algo, s
     assert worst < 0.25
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12])
 @pytest.mark.parametrize("shape", [(256, 256, 256), (300, 512, 200), (1000, 1024, 900), (513, 384, 257), (64, 128, 2048)])
 def test_every_tile_variant(pkg, oracle, variant, shape):
     """Each compiled shape of the tiled kernels (persistent and one-tile-per-workgroup),
@@ -260,6 +260,20 @@ def test_small_integers_are_exact(pkg, oracle, algo, shape):
     assert np.array_equal(C, Cref)
     ints = oracle.decode(A, 0).astype(np.int64) @ oracle.decode(B, 1).astype(np.int64).T
     assert np.array_equal(C.astype(np.int64), ints)
+
+
+@pytest.mark.parametrize("shape", [(256, 8192, 2048), (2200, 2048, 2300), (1000, 1040, 900), (512, 4096, 4096),
+                                   (128, 8192, 4096), (3000, 512, 3000), (64, 4096, 512), (77, 200, 33)])
+def test_stage4_entry_follows_the_same_plans(pkg, oracle, shape):
+    """The 4-stage entry points (gemm::GEMM4) on shapes whose plans use K slices, leftover-tile
+    slices, an overhanging K tile, the weight-streaming and the general kernel."""
+    M, K, N = shape
+    A = pkg.fill((M, K), 0, seed=0xA11CE + K + 4, dist="normal", sigma=4.0)
+    B = pkg.fill((N, K), 1, seed=0xB0B + K + 4, dist="normal", sigma=4.0)
+    C = run_gpu(pkg, A, 0, B, 1, stages=4)
+    rows = None if M * N * K < 2 ** 33 else np.arange(0, M, 4, dtype=np.int32)
+    worst = assert_within_bound(oracle, C, A, 0, B, 1, rows=rows, hw_term=K < 1024)
+    assert worst < 0.5
 
 
 def test_scratch_grows_and_is_reused_across_calls_and_streams(pkg, oracle):
