@@ -320,3 +320,44 @@ def test_back_to_back_launches_without_synchronisation(pkg, oracle):
     torch.cuda.synchronize()
     for A, B, dA, dB, out, fa in cases:
         assert_within_bound(oracle, out.cpu().numpy(), A, fa, B, 0)
+
+
+def test_random_shapes_against_the_general_kernel(pkg, oracle):
+    """Eighty seeded random shapes, pairings and stage counts through the automatic selection,
+    each compared on the GPU with the general kernel (one wave per 32 x 32 tile, no LDS, a
+    different summation order) within twice the fp32 reordering bound; the general kernel
+    itself is pinned against the CPU oracle by the tests above."""
+    import torch
+    rng = np.random.default_rng(20240611)
+    luts = [torch.from_numpy(oracle.decode(np.arange(256, dtype=np.uint8), f).astype(np.float64)).cuda() for f in (0, 1)]
+    families = set()
+    for case in range(80):
+        kind = rng.integers(0, 4)
+        if kind == 0:      # mid / large, K a multiple of 16
+            M, N, K = int(rng.integers(65, 3000)), int(rng.integers(1, 3000)), 16 * int(rng.integers(1, 300))
+        elif kind == 1:    # few rows
+            M, N, K = int(rng.integers(1, 65)), 16 * int(rng.integers(1, 400)), 128 * int(rng.integers(1, 64))
+        elif kind == 2:    # anything
+            M, N, K = int(rng.integers(1, 700)), int(rng.integers(1, 700)), int(rng.integers(1, 1500))
+        else:              # long K, few tiles
+            M, N, K = int(rng.integers(1, 600)), int(rng.integers(1, 1200)), 128 * int(rng.integers(32, 160))
+        fa, fb = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+        stages = int(rng.choice([2, 4]))
+        families.add(pkg.plan(M, K, N, stages)[0])
+        A = pkg.fill((M, K), fa, seed=1000 + case, dist="normal", sigma=2.0)
+        B = pkg.fill((N, K), fb, seed=2000 + case, dist="normal", sigma=2.0)
+        dA, dB = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+        got = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        ref = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        pkg.gemm(dA, dB, out=got, a_fmt=fa, b_fmt=fb, stages=stages)
+        pkg.gemm(dA, dB, out=ref, a_fmt=fa, b_fmt=fb, algo=ALGOS["direct"])
+        torch.cuda.synchronize()
+        S = luts[fa][dA.long()].abs() @ luts[fb][dB.long()].abs().T
+        bound = 2.0 * (2.0 * K * 2.0 ** -24) * S + 1e-30
+        err = (got.double() - ref.double()).abs()
+        assert bool(torch.isfinite(got).all()), (case, M, K, N)
+        # small K: the MFMA's internal alignment window (about 2^-13 of a block's largest product) shows
+        window = 2.0 ** -12 * S if K < 1024 else 0.0
+        ok = err <= bound + window
+        assert bool(ok.all()), (case, M, K, N, fa, fb, stages, float((err / (bound + window + 1e-30)).max()))
+    assert families == {1, 2, 3}          # the draw exercised all three kernel families
