@@ -68,6 +68,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=300)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host CPU leg")
+    ap.add_argument("--no-vendor", action="store_true", help="skip the hipBLASLt comparison (a child process)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel that FETCH_SIZE / WRITE_SIZE "
                          "counter readings are scaled by when this script runs under rocprofv3 --pmc")
@@ -177,6 +178,28 @@ def main():
         except Exception as ex:
             cpu = {"error": str(ex)[:200]}
 
+    # ---------------------------------------------------------------- vendor library beside it
+    # hipBLASLt on the same shape through the harness's comparator (a child process; per-launch
+    # events, both libraries warmed up and timed in alternating blocks).  Informational only.
+    vendor = None
+    if not args.no_vendor:
+        try:
+            import re
+            import subprocess
+            exe = os.path.join(ROOT, "tensor-core-fp8_amd", "GEMM", "out", "hipblaslt")
+            r = subprocess.run([exe, "40", "8192", "8192", "1"], capture_output=True, text=True, timeout=120)
+            mv = re.search(r"GEMM-hipblaslt-fp8: .* performance = ([0-9.eE+-]+)GFLOPS", r.stdout)
+            mo = re.search(r"GEMM-fp8gemm-fp8: .* performance = ([0-9.eE+-]+)GFLOPS", r.stdout)
+            md = re.search(r"max \|hipblaslt - fp8gemm\| = ([0-9.eE+-]+)", r.stdout)
+            if mv and mo:
+                vendor = {"library": "hipBLASLt e4m3 x e4m3 -> fp32, M=N=K=8192, per-launch events",
+                          "hipblaslt_tflops": float(mv.group(1)) / 1e3, "this_library_tflops": float(mo.group(1)) / 1e3,
+                          "max_abs_difference": float(md.group(1)) if md else None}
+            else:
+                vendor = {"error": (r.stdout + r.stderr)[-200:]}
+        except Exception as ex:
+            vendor = {"error": str(ex)[:200]}
+
     out = {
         "metric": "FP8 GEMM TFLOPS at 8192^3 e4m3 (skinny M=16 HBM GB/s in `skinny`)",
         "value": tflops,
@@ -201,6 +224,7 @@ def main():
         "skinny": skinny,
         "parity": parity,
         "cpu_baseline": cpu,
+        "vendor": vendor,
     }
     print(json.dumps(out))
 
