@@ -99,4 +99,19 @@ __device__ __forceinline__ void store_out4(void *base, size_t index, v4f v, int 
     }
 }
 
+// The same with the streaming (non-temporal) hint, for results that no kernel reads again:
+// a finished tile of C leaves through the L2 without pushing the operand panels out of it.
+__device__ __forceinline__ void store_out4_stream(void *base, size_t index, v4f v, int type)
+{
+    if (type == FP8GEMM_DEV_OUT_F32) {
+        __builtin_nontemporal_store(v, reinterpret_cast<v4f *>(static_cast<float *>(base) + index));
+    } else {
+        typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+        v2u w;
+        w[0] = out_bits16(v[0], type) | (out_bits16(v[1], type) << 16);
+        w[1] = out_bits16(v[2], type) | (out_bits16(v[3], type) << 16);
+        __builtin_nontemporal_store(w, reinterpret_cast<v2u *>(static_cast<unsigned short *>(base) + index));
+    }
+}
+
 #endif  // FP8GEMM_DEVICE_COMMON_H

@@ -111,7 +111,7 @@ hipError_t allow_lds(Kernel kernel, int bytes)
 
 template <class S, int AF, int BF>
 struct TileKernelTag {};
-template <class S, int AF, int BF, bool KOVER, bool EX>
+template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM>
 struct PtileKernelTag {};
 template <class S, int AF, int BF>
 struct SkinnyKernelTag {};
@@ -202,7 +202,21 @@ size_t ptile_scratch_bytes(const PtileWork &w, int bm, int bn)
 
 // persistent form: one workgroup per CU walks its share of the work list; the K slices'
 // partial sums go through the scratch buffer and a reduction pass
-template <class S, int AF, int BF, bool KOVER, bool EX>
+template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM>
+hipError_t launch_ptile_work(const PtileWork &w, int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
+                             float *ws, int rotate, const OutSpec &spec, hipStream_t stream)
+{
+    auto kernel = gemm_ptile_kernel<S, AF, BF, KOVER, EX, BSTREAM>;
+    hipError_t e = allow_lds<PtileKernelTag<S, AF, BF, KOVER, EX, BSTREAM>>(kernel, S::PTILE_LDS_BYTES);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * w.slots)), dim3(S::THREADS), S::PTILE_LDS_BYTES, stream,
+                       m, k, n, a, b, out, ws, w.tiles_m, w.tiles_n, w.GM, w.bulk, w.tail, w.nsplit, w.rounds, rotate, spec);
+    return hipGetLastError();
+}
+
+// STREAM_TOO: this shape is also compiled with non-temporal loads of B, used when C has a
+// single row of tiles (every byte of B is then read by exactly one workgroup)
+template <class S, int AF, int BF, bool KOVER, bool EX, bool STREAM_TOO>
 hipError_t launch_ptile_shape_k(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
                                 int nsplit, bool split_all, int rotate, const OutSpec &spec, hipStream_t stream)
 {
@@ -216,12 +230,13 @@ hipError_t launch_ptile_shape_k(int m, int k, int n, const uint8_t *a, const uin
         if (e != hipSuccess) return e;
         ws = static_cast<float *>(p);
     }
-    auto kernel = gemm_ptile_kernel<S, AF, BF, KOVER, EX>;
-    hipError_t e = allow_lds<PtileKernelTag<S, AF, BF, KOVER, EX>>(kernel, S::PTILE_LDS_BYTES);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * w.slots)), dim3(S::THREADS), S::PTILE_LDS_BYTES, stream,
-                       m, k, n, a, b, out, ws, w.tiles_m, w.tiles_n, w.GM, w.bulk, w.tail, w.nsplit, w.rounds, rotate, spec);
-    e = hipGetLastError();
+    hipError_t e;
+    if constexpr (STREAM_TOO && !KOVER) {
+        e = w.tiles_m == 1 ? launch_ptile_work<S, AF, BF, KOVER, EX, true>(w, m, k, n, a, b, out, ws, rotate, spec, stream)
+                           : launch_ptile_work<S, AF, BF, KOVER, EX, false>(w, m, k, n, a, b, out, ws, rotate, spec, stream);
+    } else {
+        e = launch_ptile_work<S, AF, BF, KOVER, EX, false>(w, m, k, n, a, b, out, ws, rotate, spec, stream);
+    }
     if (e != hipSuccess || w.nsplit == 1) return e;
     const size_t threads = (size_t)w.tail * (S::BM * S::BN / 4);
     hipLaunchKernelGGL(gemm_tile_slices_reduce_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream,
@@ -236,23 +251,23 @@ bool plain_output(const OutSpec &spec)
 
 // OVERHANG_TOO: this shape is also compiled for a K that is not a multiple of its K tile.
 // EX_TOO: ... and for the extended epilogue (scale, 16-bit output).
-template <class S, int AF, int BF, bool OVERHANG_TOO, bool EX_TOO>
+template <class S, int AF, int BF, bool OVERHANG_TOO, bool EX_TOO, bool STREAM_TOO = false>
 hipError_t launch_ptile_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
                               int nsplit, bool split_all, int rotate, const OutSpec &spec, hipStream_t stream)
 {
     const bool over = k % S::BK != 0;
     if (plain_output(spec)) {
         if (!over)
-            return launch_ptile_shape_k<S, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+            return launch_ptile_shape_k<S, AF, BF, false, false, STREAM_TOO>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
         if constexpr (OVERHANG_TOO)
-            return launch_ptile_shape_k<S, AF, BF, true, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+            return launch_ptile_shape_k<S, AF, BF, true, false, STREAM_TOO>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
         return hipErrorInvalidValue;
     }
     if constexpr (EX_TOO) {
         if (!over)
-            return launch_ptile_shape_k<S, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+            return launch_ptile_shape_k<S, AF, BF, false, true, STREAM_TOO>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
         if constexpr (OVERHANG_TOO)
-            return launch_ptile_shape_k<S, AF, BF, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+            return launch_ptile_shape_k<S, AF, BF, true, true, STREAM_TOO>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
     }
     return hipErrorInvalidValue;
 }
@@ -271,10 +286,10 @@ hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, 
     case 2: return launch_ptile_shape<TileP8, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
     case 3: return launch_tile_shape<TileS2, AF, BF>(m, k, n, a, b, static_cast<float *>(out), stream);
     case 4: return launch_tile_shape<TileS4, AF, BF>(m, k, n, a, b, static_cast<float *>(out), stream);
-    case 5: return launch_ptile_shape<TileH3, AF, BF, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
-    case 6: return launch_ptile_shape<TileQ2, AF, BF, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+    case 5: return launch_ptile_shape<TileH3, AF, BF, true, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+    case 6: return launch_ptile_shape<TileQ2, AF, BF, true, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
     case 7: return launch_tile_shape<TileS64, AF, BF>(m, k, n, a, b, static_cast<float *>(out), stream);
-    case 8: return launch_ptile_shape<TileW3, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+    case 8: return launch_ptile_shape<TileW3, AF, BF, false, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
     case 9: return launch_ptile_shape<TileT2, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
     case 10: return launch_ptile_shape<TileT4, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
     case 11: return launch_ptile_shape<TileH4, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);

@@ -52,6 +52,14 @@ __device__ __forceinline__ void buffer_load_lds_b128(v4i rsrc, uint32_t lds_addr
                  : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
                  : "m0");
 }
+// the same with the non-temporal hint, for an operand that no other workgroup reads
+__device__ __forceinline__ void buffer_load_lds_b128_stream(v4i rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen nt lds"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+                 : "m0");
+}
 #pragma clang diagnostic pop
 
 // 16-byte-per-lane LDS store whose data operand stays in accumulation registers
@@ -77,7 +85,7 @@ __device__ __forceinline__ v4i make_buffer_resource(const void *base, unsigned l
 // KOVER: the last K tile may overhang K (K % BK != 0); compiled separately so that the
 // common case carries no test for it.  EX: the output goes through `spec` (scale, fp32 /
 // bf16 / fp16); without it C receives the bare fp32 sums and `spec` is ignored.
-template <class S, int AF, int BF, bool KOVER, bool EX>
+template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM>
 __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, int N,
                                                                  const uint8_t *__restrict__ A,
                                                                  const uint8_t *__restrict__ B,
@@ -230,6 +238,8 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         }
         if (j < S::A_LOADS)
             buffer_load_lds_b128(rsA, ldsA + sbase + (uint32_t)(j * RPI * BK), voff, koff);
+        else if (BSTREAM)
+            buffer_load_lds_b128_stream(rsB, ldsB + sbase + (uint32_t)((j - S::A_LOADS) * RPI * BK), voff, koff);
         else
             buffer_load_lds_b128(rsB, ldsB + sbase + (uint32_t)((j - S::A_LOADS) * RPI * BK), voff, koff);
     };
@@ -383,7 +393,6 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
             for (int t = 0; t < STAGES - 1; ++t)
                 if (t < next_T) issue_all_loads(t, t);
         }
-
         // ---- epilogue: registers -> C -------------------------------------------
         // register q of lane (fi, fg) holds C[row0 + fi][col0 + 8*(q/4) + 4*fg + q%4]
         const int wrow0 = m0 + wm * (BM / S::WM);
@@ -424,11 +433,21 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                             lds_store_b128_acc(stg_addr + (uint32_t)(fi * ROWB + (j * 32 - c0 + 8 * q4 + 4 * fg) * 4), v);
                         }
                     if (!EX && full) {
+                        // partial sums in the scratch are read back soon (keep them cached);
+                        // C itself is not (streaming stores)
+                        const size_t first = tile_origin + (size_t)(wrow0 - m0 + i * 32 + rl) * ldo + (wcol0 - n0 + c0 + cl * 4);
+                        if (to_ws) {
 #pragma unroll
-                        for (int r0 = 0; r0 < 32; r0 += RPI_ST) {
-                            const v4f v = *reinterpret_cast<const v4f *>(stg + (r0 + rl) * ROWB + cl * 16);
-                            store_out4(tile_base, tile_origin + (size_t)(wrow0 - m0 + i * 32 + r0 + rl) * ldo + (wcol0 - n0 + c0 + cl * 4),
-                                       v, FP8GEMM_DEV_OUT_F32);
+                            for (int r0 = 0; r0 < 32; r0 += RPI_ST) {
+                                const v4f v = *reinterpret_cast<const v4f *>(stg + (r0 + rl) * ROWB + cl * 16);
+                                store_out4(tile_base, first + (size_t)r0 * ldo, v, FP8GEMM_DEV_OUT_F32);
+                            }
+                        } else {
+#pragma unroll
+                            for (int r0 = 0; r0 < 32; r0 += RPI_ST) {
+                                const v4f v = *reinterpret_cast<const v4f *>(stg + (r0 + rl) * ROWB + cl * 16);
+                                store_out4_stream(tile_base, first + (size_t)r0 * ldo, v, FP8GEMM_DEV_OUT_F32);
+                            }
                         }
                     } else {
                         // scale and convert (EX), guard (tiles that overhang C); a few rows at a time
@@ -445,7 +464,10 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                             const int lcol_ = wcol0 - n0 + c0 + cl * 4;
                             const size_t index = tile_origin + (size_t)lrow_ * ldo + lcol_;
                             if (full) {
-                                store_out4(tile_base, index, v, otype);
+                                if (to_ws)
+                                    store_out4(tile_base, index, v, otype);
+                                else
+                                    store_out4_stream(tile_base, index, v, otype);
                             } else if (m0 + lrow_ < M) {
 #pragma unroll
                                 for (int e = 0; e < 4; ++e)

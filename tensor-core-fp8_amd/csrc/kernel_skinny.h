@@ -110,9 +110,16 @@ __global__ __launch_bounds__(64) void gemm_skinny_kernel(int M, int K, int N,
         t = t >= T ? t - T : t;
 #pragma unroll
         for (int j = 0; j < S::LOADS; ++j)
-            __builtin_amdgcn_global_load_lds((const GLOBAL_AS void *)(src[j] + (size_t)t * BK),
-                                             (LDS_AS void *)(lds + stage * S::STAGE_BYTES + j * RPI * BK),
-                                             16, 0, 0);
+            // B is read exactly once: the non-temporal hint (cache-policy bit 1) lets it stream
+            // through the caches without displacing A, which every stream re-reads
+            if (j < S::A_LOADS)
+                __builtin_amdgcn_global_load_lds((const GLOBAL_AS void *)(src[j] + (size_t)t * BK),
+                                                 (LDS_AS void *)(lds + stage * S::STAGE_BYTES + j * RPI * BK),
+                                                 16, 0, 0);
+            else
+                __builtin_amdgcn_global_load_lds((const GLOBAL_AS void *)(src[j] + (size_t)t * BK),
+                                                 (LDS_AS void *)(lds + stage * S::STAGE_BYTES + j * RPI * BK),
+                                                 16, 0, 2);
     };
 
     // ---- fragment plan: lane (i = lane%16, q = lane/16) feeds row i of a 16-row
