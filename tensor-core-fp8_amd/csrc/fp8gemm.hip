@@ -390,7 +390,9 @@ SkinnyPlan plan_skinny(int m, int k, int n)
     p.tn = tn;
     p.nsplit = split;
     const int kchunk = k / split;
-    p.variant = (kchunk % 512 == 0) ? 4 : (kchunk % 256 == 0) ? 1 : 0;
+    // fat streams (64 columns) run best on 128-byte K steps in a deep ring; thinner ones want
+    // longer K steps, so that a ring stage still holds 16 KiB or more
+    p.variant = (tn == 4 && p.mt <= 3) ? 0 : (kchunk % 512 == 0) ? 4 : (kchunk % 256 == 0) ? 1 : 0;
     return p;
 }
 
