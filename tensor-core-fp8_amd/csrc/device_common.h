@@ -76,41 +76,53 @@ __device__ __forceinline__ uint32_t out_bits16(float v, int type)
     return (uint32_t)__builtin_bit_cast(unsigned short, h);
 }
 
+// Output pointers arrive as generic pointers (a choice between C and the scratch buffer, a
+// void pointer for the three output types); they always point to global memory, and saying
+// so keeps the stores from being issued as flat instructions, which also count as LDS
+// traffic in the wave's counters.
+#define FP8GEMM_GLOBAL __attribute__((address_space(1)))
+
 // element `index` of an output matrix of the given type
 __device__ __forceinline__ void store_out(void *base, size_t index, float v, int type)
 {
     if (type == FP8GEMM_DEV_OUT_F32)
-        static_cast<float *>(base)[index] = v;
+        ((FP8GEMM_GLOBAL float *)base)[index] = v;
     else
-        static_cast<unsigned short *>(base)[index] = (unsigned short)out_bits16(v, type);
+        ((FP8GEMM_GLOBAL unsigned short *)base)[index] = (unsigned short)out_bits16(v, type);
+}
+
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ v2u out_pack4(v4f v, int type)
+{
+    v2u w;
+    w[0] = out_bits16(v[0], type) | (out_bits16(v[1], type) << 16);
+    w[1] = out_bits16(v[2], type) | (out_bits16(v[3], type) << 16);
+    return w;
 }
 
 // four consecutive elements starting at `index` (index % 4 == 0, 16-byte aligned base)
 __device__ __forceinline__ void store_out4(void *base, size_t index, v4f v, int type)
 {
-    if (type == FP8GEMM_DEV_OUT_F32) {
-        *reinterpret_cast<v4f *>(static_cast<float *>(base) + index) = v;
-    } else {
-        typedef unsigned int v2u __attribute__((ext_vector_type(2)));
-        v2u w;
-        w[0] = out_bits16(v[0], type) | (out_bits16(v[1], type) << 16);
-        w[1] = out_bits16(v[2], type) | (out_bits16(v[3], type) << 16);
-        *reinterpret_cast<v2u *>(static_cast<unsigned short *>(base) + index) = w;
-    }
+    if (type == FP8GEMM_DEV_OUT_F32)
+        *(FP8GEMM_GLOBAL v4f *)((FP8GEMM_GLOBAL float *)base + index) = v;
+    else
+        *(FP8GEMM_GLOBAL v2u *)((FP8GEMM_GLOBAL unsigned short *)base + index) = out_pack4(v, type);
 }
 
 // The same with the streaming (non-temporal) hint, for results that no kernel reads again:
 // a finished tile of C leaves through the L2 without pushing the operand panels out of it.
+// Written as assembly: where a branch chooses between a plain and a non-temporal store of
+// the same value, the optimizer merges the two into one plain store and the hint is lost.
 __device__ __forceinline__ void store_out4_stream(void *base, size_t index, v4f v, int type)
 {
     if (type == FP8GEMM_DEV_OUT_F32) {
-        __builtin_nontemporal_store(v, reinterpret_cast<v4f *>(static_cast<float *>(base) + index));
+        FP8GEMM_GLOBAL v4f *p = (FP8GEMM_GLOBAL v4f *)((FP8GEMM_GLOBAL float *)base + index);
+        asm volatile("global_store_dwordx4 %0, %1, off nt" : : "v"(p), "v"(v) : "memory");
     } else {
-        typedef unsigned int v2u __attribute__((ext_vector_type(2)));
-        v2u w;
-        w[0] = out_bits16(v[0], type) | (out_bits16(v[1], type) << 16);
-        w[1] = out_bits16(v[2], type) | (out_bits16(v[3], type) << 16);
-        __builtin_nontemporal_store(w, reinterpret_cast<v2u *>(static_cast<unsigned short *>(base) + index));
+        FP8GEMM_GLOBAL v2u *p = (FP8GEMM_GLOBAL v2u *)((FP8GEMM_GLOBAL unsigned short *)base + index);
+        const v2u w = out_pack4(v, type);
+        asm volatile("global_store_dwordx2 %0, %1, off nt" : : "v"(p), "v"(w) : "memory");
     }
 }
 

@@ -62,6 +62,16 @@ __device__ __forceinline__ void buffer_load_lds_b128_stream(v4i rsrc, uint32_t l
 }
 #pragma clang diagnostic pop
 
+// f(integral_constant<int, I>) for I = FIRST .. LAST-1, unrolled at compile time
+template <int FIRST, int LAST, class F>
+__device__ __forceinline__ void static_for(F &f)
+{
+    if constexpr (FIRST < LAST) {
+        f(std::integral_constant<int, FIRST>{});
+        static_for<FIRST + 1, LAST>(f);
+    }
+}
+
 // 16-byte-per-lane LDS store whose data operand stays in accumulation registers
 // (the MFMA results live there; copying all of them to ordinary vector registers
 // first would need 256 more registers per lane).
@@ -421,61 +431,79 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
             uint8_t *stg = lds + S::EP_OFFSET + wave * (32 * ROWB);
             const uint32_t stg_addr = lds_base + (uint32_t)(S::EP_OFFSET + wave * (32 * ROWB));
             const int rl = lane / LPR, cl = lane % LPR;
+            constexpr int CHUNKS = TN * 32 / EP;                 // column chunks of a 32-row block
+            constexpr int NSTEP = TM * CHUNKS;                   // strips to stage
+            constexpr int NR = 32 / RPI_ST;                      // store instructions per strip
+            // strip st = rows 32*(st / CHUNKS) .., columns EP*(st % CHUNKS) .. of the wave's part
+            auto stage_strip = [&](auto stc) __attribute__((always_inline)) {
+                constexpr int ST = decltype(stc)::value;
+                constexpr int i = ST / CHUNKS, c0 = (ST % CHUNKS) * EP;
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+                for (int j = c0 / 32; j < (c0 + EP) / 32; ++j)
 #pragma unroll
-                for (int c0 = 0; c0 < TN * 32; c0 += EP) {
+                    for (int q4 = 0; q4 < 4; ++q4) {
+                        v4f v = {acc[i][j][4 * q4], acc[i][j][4 * q4 + 1], acc[i][j][4 * q4 + 2], acc[i][j][4 * q4 + 3]};
+                        lds_store_b128_acc(stg_addr + (uint32_t)(fi * ROWB + (j * 32 - c0 + 8 * q4 + 4 * fg) * 4), v);
+                    }
+            };
+            auto drain_strip = [&](auto stc) __attribute__((always_inline)) {
+                constexpr int ST = decltype(stc)::value;
+                constexpr int i = ST / CHUNKS, c0 = (ST % CHUNKS) * EP;
+                const int lrow0 = wrow0 - m0 + i * 32 + rl;          // inside the tile
+                const int lcol_ = wcol0 - n0 + c0 + cl * 4;
+                const size_t first = tile_origin + (size_t)lrow0 * ldo + lcol_;
+                if (full) {
+                    // All reads of the strip go out back to back, then the next strip is staged
+                    // (the LDS serves one wave's instructions in order, so those writes land after
+                    // these reads), then the stores follow as the data arrive: one LDS round trip
+                    // per strip instead of one per store.
+                    v4f buf[NR];
 #pragma unroll
-                    for (int j = c0 / 32; j < (c0 + EP) / 32; ++j)
+                    for (int u = 0; u < NR; ++u)
+                        buf[u] = *reinterpret_cast<const v4f *>(stg + (u * RPI_ST + rl) * ROWB + cl * 16);
+                    if constexpr (ST + 1 < NSTEP) stage_strip(std::integral_constant<int, ST + 1>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (EX) {
 #pragma unroll
-                        for (int q4 = 0; q4 < 4; ++q4) {
-                            v4f v = {acc[i][j][4 * q4], acc[i][j][4 * q4 + 1], acc[i][j][4 * q4 + 2], acc[i][j][4 * q4 + 3]};
-                            lds_store_b128_acc(stg_addr + (uint32_t)(fi * ROWB + (j * 32 - c0 + 8 * q4 + 4 * fg) * 4), v);
-                        }
-                    if (!EX && full) {
-                        // partial sums in the scratch are read back soon (keep them cached);
-                        // C itself is not (streaming stores)
-                        const size_t first = tile_origin + (size_t)(wrow0 - m0 + i * 32 + rl) * ldo + (wcol0 - n0 + c0 + cl * 4);
-                        if (to_ws) {
-#pragma unroll
-                            for (int r0 = 0; r0 < 32; r0 += RPI_ST) {
-                                const v4f v = *reinterpret_cast<const v4f *>(stg + (r0 + rl) * ROWB + cl * 16);
-                                store_out4(tile_base, first + (size_t)r0 * ldo, v, FP8GEMM_DEV_OUT_F32);
-                            }
-                        } else {
-#pragma unroll
-                            for (int r0 = 0; r0 < 32; r0 += RPI_ST) {
-                                const v4f v = *reinterpret_cast<const v4f *>(stg + (r0 + rl) * ROWB + cl * 16);
-                                store_out4_stream(tile_base, first + (size_t)r0 * ldo, v, FP8GEMM_DEV_OUT_F32);
-                            }
-                        }
-                    } else {
-                        // scale and convert (EX), guard (tiles that overhang C); a few rows at a time
-#pragma unroll 2
-                        for (int r0 = 0; r0 < 32; r0 += RPI_ST) {
-                            v4f v = *reinterpret_cast<const v4f *>(stg + (r0 + rl) * ROWB + cl * 16);
-                            if (EX) {
-                                v[0] *= oscale;
-                                v[1] *= oscale;
-                                v[2] *= oscale;
-                                v[3] *= oscale;
-                            }
-                            const int lrow_ = wrow0 - m0 + i * 32 + r0 + rl;       // inside the tile
-                            const int lcol_ = wcol0 - n0 + c0 + cl * 4;
-                            const size_t index = tile_origin + (size_t)lrow_ * ldo + lcol_;
-                            if (full) {
-                                if (to_ws)
-                                    store_out4(tile_base, index, v, otype);
-                                else
-                                    store_out4_stream(tile_base, index, v, otype);
-                            } else if (m0 + lrow_ < M) {
-#pragma unroll
-                                for (int e = 0; e < 4; ++e)
-                                    if (n0 + lcol_ + e < N) store_out(tile_base, index + e, v[e], otype);
-                            }
+                        for (int u = 0; u < NR; ++u) {
+                            buf[u][0] *= oscale;
+                            buf[u][1] *= oscale;
+                            buf[u][2] *= oscale;
+                            buf[u][3] *= oscale;
                         }
                     }
+                    // partial sums in the scratch are read back soon (keep them cached);
+                    // C itself is not (streaming stores)
+                    if (to_ws) {
+#pragma unroll
+                        for (int u = 0; u < NR; ++u) store_out4(tile_base, first + (size_t)(u * RPI_ST) * ldo, buf[u], otype);
+                    } else {
+#pragma unroll
+                        for (int u = 0; u < NR; ++u) store_out4_stream(tile_base, first + (size_t)(u * RPI_ST) * ldo, buf[u], otype);
+                    }
+                } else {
+                    // a tile that overhangs C: every element store guarded, a few rows at a time
+#pragma unroll 2
+                    for (int r0 = 0; r0 < 32; r0 += RPI_ST) {
+                        v4f v = *reinterpret_cast<const v4f *>(stg + (r0 + rl) * ROWB + cl * 16);
+                        if (EX) {
+                            v[0] *= oscale;
+                            v[1] *= oscale;
+                            v[2] *= oscale;
+                            v[3] *= oscale;
+                        }
+                        const size_t index = first + (size_t)r0 * ldo;
+                        if (m0 + lrow0 + r0 < M) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                if (n0 + lcol_ + e < N) store_out(tile_base, index + e, v[e], otype);
+                        }
+                    }
+                    if constexpr (ST + 1 < NSTEP) stage_strip(std::integral_constant<int, ST + 1>{});
                 }
+            };
+            stage_strip(std::integral_constant<int, 0>{});
+            static_for<0, NSTEP>(drain_strip);
         }
         tile_m = next_m;
         tile_n = next_n;
