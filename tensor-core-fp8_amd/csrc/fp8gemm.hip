@@ -25,6 +25,7 @@ constexpr int kMaxDevices = 64;
 // ------------------------------------------------------------------ variants
 // Tiled kernel shapes: <BM, BN, BK, waves_m, waves_n, stages, swizzle>.
 using TileP2 = TileShape<256, 256, 128, 2, 2, 2, 3>;  // persistent, 2 x 64 KiB ring, 128x128 per wave
+using TileP2h = TileShape<256, 256, 128, 2, 2, 2, 3, true>;   // the same on v_mfma_f32_16x16x128_f8f6f4
 using TileP4 = TileShape<256, 256, 64, 2, 2, 4, 2>;   // persistent, 4 x 32 KiB ring
 using TileP8 = TileShape<256, 256, 128, 2, 4, 2, 3>;  // persistent, 8 waves, 128x64 per wave
 using TileS2 = TileShape<128, 128, 128, 2, 2, 2, 3>;  // one tile per workgroup, for small problems
@@ -38,7 +39,7 @@ using TileT2 = TileShape<192, 256, 128, 2, 2, 2, 3>;  // persistent, three-quart
 using TileT4 = TileShape<192, 256, 64, 2, 2, 4, 2>;
 using TileH4 = TileShape<128, 256, 64, 2, 2, 4, 2>;
 using TileQ4 = TileShape<128, 128, 64, 2, 2, 4, 2>;
-constexpr int kNumTileVariants = 13;              // 0 P2, 1 P4, 2 P8, 3 S2, 4 S4, 5 H3, 6 Q2, 7 S64, 8 W3, 9 T2, 10 T4, 11 H4, 12 Q4
+constexpr int kNumTileVariants = 14;              // 0 P2, 1 P4, 2 P8, 3 S2, 4 S4, 5 H3, 6 Q2, 7 S64, 8 W3, 9 T2, 10 T4, 11 H4, 12 Q4, 13 P2h
 
 // Skinny kernel shapes: <MT, TN, BK, stages>.
 template <int MT, int TN>
@@ -272,6 +273,13 @@ hipError_t launch_ptile_shape(int m, int k, int n, const uint8_t *a, const uint8
     return hipErrorInvalidValue;
 }
 
+// The 16x16x128 form of the 256 x 256 tile walks K in pairs of 128-byte K tiles: every work
+// item (a tile, or one of its nsplit K slices) must hold an even number of them.
+bool p2h_ok(int k, int nsplit)
+{
+    return k % 128 == 0 && (k / 128) % (2 * nsplit) == 0;
+}
+
 template <int AF, int BF>
 hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
                        int variant, int nsplit, bool split_all, int rotate, const OutSpec &spec, hipStream_t stream)
@@ -294,6 +302,9 @@ hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, 
     case 10: return launch_ptile_shape<TileT4, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
     case 11: return launch_ptile_shape<TileH4, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
     case 12: return launch_ptile_shape<TileQ4, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+    case 13:
+        if (!p2h_ok(k, nsplit)) return hipErrorInvalidValue;
+        return launch_ptile_shape<TileP2h, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
     default: return hipErrorInvalidValue;
     }
 }

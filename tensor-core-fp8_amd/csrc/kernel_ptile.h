@@ -281,115 +281,204 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         }
         const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-        v16f acc[TM][TN];
+        // accumulators: TM x TN blocks of 32 x 32 (16 registers each), or twice as many
+        // blocks of 16 x 16 each way (4 registers each); 256 registers per lane either way
+        using AccT = std::conditional_t<S::MF16, v4f, v16f>;
+        constexpr int AM = S::MF16 ? 2 * TM : TM, AN = S::MF16 ? 2 * TN : TN;
+        AccT acc[AM][AN];
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < AM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
+            for (int j = 0; j < AN; ++j)
 #pragma unroll
-                for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.0f;
+                for (int q = 0; q < (S::MF16 ? 4 : 16); ++q) acc[i][j][q] = 0.0f;
 
-        // fragment sets: frag[p][0..TM-1] = A blocks, frag[p][TM..TM+TN-1] = B blocks
-        v4i frag[2][TM + TN][2];
-        // read number q (0 .. NREADS-1) of K step ks of ring slot `stage` into set p.
-        // Order: B0, A0, B1 .. B(TN-1), A1 .. A(TM-1), the order the MFMAs need them.
-        auto issue_read = [&](auto pc, int q, int stage, int ks) {
-            constexpr int P = decltype(pc)::value;
-            const int f = q >> 1, h = q & 1;
-            int idx;           // index into frag[P]
-            if (f == 0) idx = TM;
-            else if (f == 1) idx = 0;
-            else if (f <= TN) idx = TM + f - 1;
-            else idx = f - TN;
-            const uint32_t rowbase = idx < TM ? a_base + (uint32_t)(idx * 32 * BK) : b_base + (uint32_t)((idx - TM) * 32 * BK);
-            const uint8_t *p = lds + stage * S::STAGE_BYTES + rowbase + frag_off[ks][h];
-            frag[P][idx][h] = *reinterpret_cast<const v4i *>(p);
-        };
+        if constexpr (!S::MF16) {
+            // fragment sets: frag[p][0..TM-1] = A blocks, frag[p][TM..TM+TN-1] = B blocks
+            v4i frag[2][TM + TN][2];
+            // read number q (0 .. NREADS-1) of K step ks of ring slot `stage` into set p.
+            // Order: B0, A0, B1 .. B(TN-1), A1 .. A(TM-1), the order the MFMAs need them.
+            auto issue_read = [&](auto pc, int q, int stage, int ks) {
+                constexpr int P = decltype(pc)::value;
+                const int f = q >> 1, h = q & 1;
+                int idx;           // index into frag[P]
+                if (f == 0) idx = TM;
+                else if (f == 1) idx = 0;
+                else if (f <= TN) idx = TM + f - 1;
+                else idx = f - TN;
+                const uint32_t rowbase = idx < TM ? a_base + (uint32_t)(idx * 32 * BK) : b_base + (uint32_t)((idx - TM) * 32 * BK);
+                const uint8_t *p = lds + stage * S::STAGE_BYTES + rowbase + frag_off[ks][h];
+                frag[P][idx][h] = *reinterpret_cast<const v4i *>(p);
+            };
 
-        // K tile 0 must have landed before the first fragment read.  The stores of
-        // the previous tile's epilogue are still in flight and share the counter
-        // with the loads (and may retire out of order with them), so wait for all.
-        wait_vmcnt<0>();
-        __syncthreads();
-        if (STAGES - 1 < T) issue_all_loads(STAGES - 1, STAGES - 1);
-        using I0 = std::integral_constant<int, 0>;
-        using I1 = std::integral_constant<int, 1>;
+            // K tile 0 must have landed before the first fragment read.  The stores of
+            // the previous tile's epilogue are still in flight and share the counter
+            // with the loads (and may retire out of order with them), so wait for all.
+            wait_vmcnt<0>();
+            __syncthreads();
+            if (STAGES - 1 < T) issue_all_loads(STAGES - 1, STAGES - 1);
+            using I0 = std::integral_constant<int, 0>;
+            using I1 = std::integral_constant<int, 1>;
 #pragma unroll
-        for (int q = 0; q < NREADS; ++q) issue_read(I0{}, q, 0, 0);
+            for (int q = 0; q < NREADS; ++q) issue_read(I0{}, q, 0, 0);
 
-        // One K step.  P = parity of the global step (which fragment set feeds the
-        // MFMAs), KS = K step inside the K tile, next = a further K tile follows,
-        // load = a K tile STAGES ahead exists and is fetched now (both uniform; the
-        // steady-state loop passes constants so that no branch is left in it).
-        auto kstep = [&](auto pc, auto sc, const bool next, const bool load, int t) {
-            constexpr int P = decltype(pc)::value;
-            constexpr int KS = decltype(sc)::value;
-            using PN = std::integral_constant<int, P ^ 1>;
-            const int stage = t % STAGES;
-            constexpr bool last_ks = (KS + 1 == KSTEPS);
-            int rstage = stage, rks = KS + 1;
-            bool reads = true;
-            if (last_ks) {
-                rstage = (t + 1) % STAGES;
-                rks = 0;
-                reads = next;
+            // One K step.  P = parity of the global step (which fragment set feeds the
+            // MFMAs), KS = K step inside the K tile, next = a further K tile follows,
+            // load = a K tile STAGES ahead exists and is fetched now (both uniform; the
+            // steady-state loop passes constants so that no branch is left in it).
+            auto kstep = [&](auto pc, auto sc, const bool next, const bool load, int t) {
+                constexpr int P = decltype(pc)::value;
+                constexpr int KS = decltype(sc)::value;
+                using PN = std::integral_constant<int, P ^ 1>;
+                const int stage = t % STAGES;
+                constexpr bool last_ks = (KS + 1 == KSTEPS);
+                int rstage = stage, rks = KS + 1;
+                bool reads = true;
+                if (last_ks) {
+                    rstage = (t + 1) % STAGES;
+                    rks = 0;
+                    reads = next;
+                    if (next) {
+                        // every fragment read of K tile t has been issued; once they have
+                        // returned this wave no longer needs the ring slot
+                        wait_lgkmcnt0();
+                        if (load)
+                            wait_vmcnt<S::LOADS *(STAGES - 2)>();
+                        else
+                            wait_vmcnt<0>();
+                        __syncthreads();
+                    }
+                }
+                // reads per MFMA slot and loads per MFMA slot, rounded up
+                constexpr int RD_PER = (NREADS + NMFMA - 1) / NMFMA;
+                constexpr int LD_PER = (S::LOADS + NMFMA - 1) / NMFMA;
+#pragma unroll
+                for (int m = 0; m < NMFMA; ++m) {
+                    const int i = m / TN, j = m % TN;
+                    acc[i][j] = mfma_32x32x64<BF, AF>(pack8(frag[P][TM + j][0], frag[P][TM + j][1]),
+                                                      pack8(frag[P][i][0], frag[P][i][1]), acc[i][j]);
+                    if (last_ks && load) {
+#pragma unroll
+                        for (int u = 0; u < LD_PER; ++u)
+                            if (m * LD_PER + u < S::LOADS) issue_load(m * LD_PER + u, t + STAGES, stage);
+                    }
+                    if (reads) {
+#pragma unroll
+                        for (int u = 0; u < RD_PER; ++u)
+                            if (m * RD_PER + u < NREADS) issue_read(PN{}, m * RD_PER + u, rstage, rks % KSTEPS);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            };
+            // K tiles [0, T-STAGES) fetch ahead, [T-STAGES, T-1) only consume, T-1 is last
+            const int t_load_end = T - STAGES > 0 ? T - STAGES : 0;
+            if (KSTEPS == 2) {
+                int t = 0;
+                for (; t < t_load_end; ++t) {
+                    kstep(I0{}, I0{}, true, true, t);
+                    kstep(I1{}, I1{}, true, true, t);
+                }
+                for (; t < T; ++t) {
+                    kstep(I0{}, I0{}, t + 1 < T, false, t);
+                    kstep(I1{}, I1{}, t + 1 < T, false, t);
+                }
+            } else {
+                // one K step per K tile: the fragment sets alternate from K tile to K tile, so
+                // K tiles go in pairs (an odd count ends on a single one)
+                const int t_pair_end = t_load_end & ~1;
+                int t = 0;
+                for (; t < t_pair_end; t += 2) {
+                    kstep(I0{}, I0{}, true, true, t);
+                    kstep(I1{}, I0{}, true, true, t + 1);
+                }
+                for (; t < T; t += 2) {
+                    kstep(I0{}, I0{}, t + 1 < T, t < t_load_end, t);
+                    if (t + 1 < T) kstep(I1{}, I0{}, t + 2 < T, t + 1 < t_load_end, t + 1);
+                }
+            }
+
+        } else {
+            // ---- v_mfma_f32_16x16x128_f8f6f4: one MFMA K step per K tile -------------
+            // Lane (hi = lane % 16, hq = lane / 16) feeds row hi of a 16-row block with K
+            // quarter hq (chunks 2*hq, 2*hq + 1 of the row).  The B fragments of a K tile
+            // (8 blocks, 64 registers) stay resident for its 64 MFMAs and are double
+            // buffered across K tiles; the A fragments stream through: blocks 1..7 are read
+            // during block rows 0..3 (two reads in every four MFMAs), so that every read of the
+            // ring slot has been issued by the middle of the K tile.  There the one barrier of the K tile sits: the next K
+            // tile has landed (its B fragments and first A fragment are read during block rows
+            // 4..7) and the slot just read is free for the K tile after that.
+            static_assert(STAGES == 2 && KSTEPS == 2 && TM == 4 && TN == 4, "the 16x16x128 schedule is written for 128 x 128 per wave, 128-byte K tiles, two ring slots");
+            const int hi = lane & 15, hq = lane >> 4;
+            const int hsw = tile_swizzle<BK, S::SWZ>(hi);             // same for rows hi + 16 * block
+            const uint32_t hoff0 = (uint32_t)(((2 * hq) ^ hsw) * 16), hoff1 = (uint32_t)(((2 * hq + 1) ^ hsw) * 16);
+            const uint32_t ha_base = (uint32_t)(wm * (BM / S::WM) + hi) * BK;
+            const uint32_t hb_base = (uint32_t)(BM * BK) + (uint32_t)(wn * (BN / S::WN) + hi) * BK;
+            v4i fb[2][8][2], fa[5][2];       // A block i lives in fa[i % 5]
+            auto read_a = [&](int blk, int h, int stage) __attribute__((always_inline)) {
+                fa[blk % 5][h] = *reinterpret_cast<const v4i *>(lds + stage * S::STAGE_BYTES + ha_base + (uint32_t)(blk * 16 * BK) + (h ? hoff1 : hoff0));
+            };
+            auto read_b = [&](auto pc, int blk, int h, int stage) __attribute__((always_inline)) {
+                constexpr int P = decltype(pc)::value;
+                fb[P][blk][h] = *reinterpret_cast<const v4i *>(lds + stage * S::STAGE_BYTES + hb_base + (uint32_t)(blk * 16 * BK) + (h ? hoff1 : hoff0));
+            };
+            using I0 = std::integral_constant<int, 0>;
+            using I1 = std::integral_constant<int, 1>;
+            wait_vmcnt<0>();
+            __syncthreads();
+            if (1 < T) issue_all_loads(1, 1);
+#pragma unroll
+            for (int q = 0; q < 16; ++q) read_b(I0{}, q >> 1, q & 1, 0);
+            read_a(0, 0, 0);
+            read_a(0, 1, 0);
+
+            // K tile t with B fragment set P; next: a further K tile follows; load: the K tile
+            // after that exists and is fetched now (both uniform)
+            auto ktile = [&](auto pc, const bool next, const bool load, int t) __attribute__((always_inline)) {
+                constexpr int P = decltype(pc)::value;
+                using PN = std::integral_constant<int, P ^ 1>;
+                const int stage = t & 1, nstage = stage ^ 1;
+#pragma unroll
+                for (int m = 0; m < 32; ++m) {
+                    const int i = m >> 3, j = m & 7;
+                    acc[i][j] = mfma_16x16x128<BF, AF>(pack8(fb[P][j][0], fb[P][j][1]), pack8(fa[i % 5][0], fa[i % 5][1]), acc[i][j]);
+                    // block b goes to the place of block b - 5, whose block row is over by then
+                    if (m < 28 && (m & 3) < 2) read_a(1 + (m >> 2), m & 1, stage);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
                 if (next) {
-                    // every fragment read of K tile t has been issued; once they have
-                    // returned this wave no longer needs the ring slot
                     wait_lgkmcnt0();
-                    if (load)
-                        wait_vmcnt<S::LOADS *(STAGES - 2)>();
-                    else
-                        wait_vmcnt<0>();
+                    wait_vmcnt<0>();
                     __syncthreads();
                 }
-            }
-            // reads per MFMA slot and loads per MFMA slot, rounded up
-            constexpr int RD_PER = (NREADS + NMFMA - 1) / NMFMA;
-            constexpr int LD_PER = (S::LOADS + NMFMA - 1) / NMFMA;
 #pragma unroll
-            for (int m = 0; m < NMFMA; ++m) {
-                const int i = m / TN, j = m % TN;
-                acc[i][j] = mfma_32x32x64<BF, AF>(pack8(frag[P][TM + j][0], frag[P][TM + j][1]),
-                                                  pack8(frag[P][i][0], frag[P][i][1]), acc[i][j]);
-                if (last_ks && load) {
-#pragma unroll
-                    for (int u = 0; u < LD_PER; ++u)
-                        if (m * LD_PER + u < S::LOADS) issue_load(m * LD_PER + u, t + STAGES, stage);
+                for (int m = 0; m < 32; ++m) {
+                    const int i = 4 + (m >> 3), j = m & 7;
+                    acc[i][j] = mfma_16x16x128<BF, AF>(pack8(fb[P][j][0], fb[P][j][1]), pack8(fa[i % 5][0], fa[i % 5][1]), acc[i][j]);
+                    // a 16x16x128 MFMA lasts 32 clocks: room for about one memory instruction
+                    // beside it.  Even slots take the 16 loads of the K tile after next, odd
+                    // slots the 16 reads of the next B fragments, slots 28 and 30 also the
+                    // two reads of the next first A fragment.
+                    if ((m & 1) == 0) {
+                        if (load && (m >> 1) < S::LOADS) issue_load(m >> 1, t + 2, stage);
+                        if (next && m >= 28) read_a(0, (m >> 1) & 1, nstage);
+                    } else if (next) {
+                        read_b(PN{}, m >> 2, (m >> 1) & 1, nstage);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-                if (reads) {
-#pragma unroll
-                    for (int u = 0; u < RD_PER; ++u)
-                        if (m * RD_PER + u < NREADS) issue_read(PN{}, m * RD_PER + u, rstage, rks % KSTEPS);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        };
-        // K tiles [0, T-STAGES) fetch ahead, [T-STAGES, T-1) only consume, T-1 is last
-        const int t_load_end = T - STAGES > 0 ? T - STAGES : 0;
-        if (KSTEPS == 2) {
+            };
+            static_assert(S::LOADS <= 16, "the loads of a K tile are issued beside every other MFMA of block rows 4..7");
+            // T is even here (the host sends other K-tile counts to the 32x32x64 kernel): K tiles
+            // go in pairs, one per B fragment set, and the last pair is written out so that no
+            // branch surrounds a K tile (all 256 accumulation registers are taken; a copy of an
+            // accumulator at a join would have nowhere to go)
             int t = 0;
-            for (; t < t_load_end; ++t) {
-                kstep(I0{}, I0{}, true, true, t);
-                kstep(I1{}, I1{}, true, true, t);
+            for (; t < T - 2; t += 2) {
+                ktile(I0{}, true, true, t);
+                ktile(I1{}, true, true, t + 1);
             }
-            for (; t < T; ++t) {
-                kstep(I0{}, I0{}, t + 1 < T, false, t);
-                kstep(I1{}, I1{}, t + 1 < T, false, t);
-            }
-        } else {
-            // one K step per K tile: the fragment sets alternate from K tile to K tile, so
-            // K tiles go in pairs (an odd count ends on a single one)
-            const int t_pair_end = t_load_end & ~1;
-            int t = 0;
-            for (; t < t_pair_end; t += 2) {
-                kstep(I0{}, I0{}, true, true, t);
-                kstep(I1{}, I0{}, true, true, t + 1);
-            }
-            for (; t < T; t += 2) {
-                kstep(I0{}, I0{}, t + 1 < T, t < t_load_end, t);
-                if (t + 1 < T) kstep(I1{}, I0{}, t + 2 < T, t + 1 < t_load_end, t + 1);
-            }
+            ktile(I0{}, true, false, t);
+            ktile(I1{}, false, false, t + 1);
         }
 
         // all waves are done reading LDS for this tile before the ring is reused
@@ -438,13 +527,22 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
             auto stage_strip = [&](auto stc) __attribute__((always_inline)) {
                 constexpr int ST = decltype(stc)::value;
                 constexpr int i = ST / CHUNKS, c0 = (ST % CHUNKS) * EP;
+                if constexpr (!S::MF16) {
 #pragma unroll
-                for (int j = c0 / 32; j < (c0 + EP) / 32; ++j)
+                    for (int j = c0 / 32; j < (c0 + EP) / 32; ++j)
 #pragma unroll
-                    for (int q4 = 0; q4 < 4; ++q4) {
-                        v4f v = {acc[i][j][4 * q4], acc[i][j][4 * q4 + 1], acc[i][j][4 * q4 + 2], acc[i][j][4 * q4 + 3]};
-                        lds_store_b128_acc(stg_addr + (uint32_t)(fi * ROWB + (j * 32 - c0 + 8 * q4 + 4 * fg) * 4), v);
-                    }
+                        for (int q4 = 0; q4 < 4; ++q4) {
+                            v4f v = {acc[i][j][4 * q4], acc[i][j][4 * q4 + 1], acc[i][j][4 * q4 + 2], acc[i][j][4 * q4 + 3]};
+                            lds_store_b128_acc(stg_addr + (uint32_t)(fi * ROWB + (j * 32 - c0 + 8 * q4 + 4 * fg) * 4), v);
+                        }
+                } else {
+                    // lane (lane % 16, lane / 16) of block (ib, jb) holds C[16*ib + lane%16][16*jb + 4*(lane/16) .. +3]
+#pragma unroll
+                    for (int ib = 2 * i; ib < 2 * i + 2; ++ib)
+#pragma unroll
+                        for (int jb = c0 / 16; jb < (c0 + EP) / 16; ++jb)
+                            lds_store_b128_acc(stg_addr + (uint32_t)((16 * (ib & 1) + (lane & 15)) * ROWB + (16 * jb - c0 + 4 * (lane >> 4)) * 4), acc[ib][jb]);
+                }
             };
             auto drain_strip = [&](auto stc) __attribute__((always_inline)) {
                 constexpr int ST = decltype(stc)::value;

@@ -40,10 +40,13 @@ __device__ __forceinline__ int tile_swizzle(int row)
     return ((row % CH) ^ ((row / CH) & 1)) % CH;
 }
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int SWZ_>
+// MF16_: the persistent kernel computes with v_mfma_f32_16x16x128_f8f6f4 (64 blocks of
+// 16 x 16 per wave) instead of v_mfma_f32_32x32x64_f8f6f4 (16 blocks of 32 x 32)
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, int SWZ_, bool MF16_ = false>
 struct TileShape {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
     static constexpr int STAGES = STAGES_, SWZ = SWZ_;
+    static constexpr bool MF16 = MF16_;
     static constexpr int NW = WM * WN;
     static constexpr int THREADS = NW * 64;
     static constexpr int CH = BK / 16;            // 16-byte chunks per row
