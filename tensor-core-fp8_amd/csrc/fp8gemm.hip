@@ -494,6 +494,10 @@ TilePlan plan_tile(int m, int k, int n, int stages)
     // K-walk rotation: per tile column while A is small enough to stay in an XCD's L2
     // next to the B rows in flight, else per XCD and round
     best.rotate = ((size_t)m * k <= ((size_t)2 << 20)) ? 1 : 2;
+    // the 256 x 256 tile runs on the 16x16x128 MFMA where its K walk allows it: the same
+    // tile, work list and traffic, about 8 % less energy per flop -- and the 8192^3-class
+    // shapes run at the board's power limit
+    if (best.variant == 0 && p2h_ok(k, best.nsplit)) best.variant = 13;
     return best;
 }
 
@@ -501,7 +505,7 @@ size_t tile_plan_scratch_bytes(int m, int n, const TilePlan &p)
 {
     if (p.nsplit <= 1) return 0;
     for (const PtileCost &c : kPtileCosts)
-        if (c.variant == p.variant || c.variant4 == p.variant) {
+        if (c.variant == p.variant || c.variant4 == p.variant || (c.variant == 0 && p.variant == 13)) {
             const PtileWork w = ptile_work(m, n, c.bm, c.bn, p.nsplit, p.split_all);
             return w.ok ? ptile_scratch_bytes(w, c.bm, c.bn) : 0;
         }

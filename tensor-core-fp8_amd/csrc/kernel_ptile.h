@@ -413,9 +413,9 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
             const uint32_t hoff0 = (uint32_t)(((2 * hq) ^ hsw) * 16), hoff1 = (uint32_t)(((2 * hq + 1) ^ hsw) * 16);
             const uint32_t ha_base = (uint32_t)(wm * (BM / S::WM) + hi) * BK;
             const uint32_t hb_base = (uint32_t)(BM * BK) + (uint32_t)(wn * (BN / S::WN) + hi) * BK;
-            v4i fb[2][8][2], fa[5][2];       // A block i lives in fa[i % 5]
+            v4i fb[2][8][2], fa[6][2];       // A block 0 lives in fa[5], block i > 0 in fa[(i - 1) % 5]
             auto read_a = [&](int blk, int h, int stage) __attribute__((always_inline)) {
-                fa[blk % 5][h] = *reinterpret_cast<const v4i *>(lds + stage * S::STAGE_BYTES + ha_base + (uint32_t)(blk * 16 * BK) + (h ? hoff1 : hoff0));
+                fa[blk == 0 ? 5 : (blk - 1) % 5][h] = *reinterpret_cast<const v4i *>(lds + stage * S::STAGE_BYTES + ha_base + (uint32_t)(blk * 16 * BK) + (h ? hoff1 : hoff0));
             };
             auto read_b = [&](auto pc, int blk, int h, int stage) __attribute__((always_inline)) {
                 constexpr int P = decltype(pc)::value;
@@ -440,8 +440,8 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
 #pragma unroll
                 for (int m = 0; m < 32; ++m) {
                     const int i = m >> 3, j = m & 7;
-                    acc[i][j] = mfma_16x16x128<BF, AF>(pack8(fb[P][j][0], fb[P][j][1]), pack8(fa[i % 5][0], fa[i % 5][1]), acc[i][j]);
-                    // block b goes to the place of block b - 5, whose block row is over by then
+                    acc[i][j] = mfma_16x16x128<BF, AF>(pack8(fb[P][j][0], fb[P][j][1]), pack8(fa[i == 0 ? 5 : (i - 1) % 5][0], fa[i == 0 ? 5 : (i - 1) % 5][1]), acc[i][j]);
+                    // block b > 5 goes to the place of block b - 5, whose block row is over by then
                     if (m < 28 && (m & 3) < 2) read_a(1 + (m >> 2), m & 1, stage);
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -453,14 +453,14 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
 #pragma unroll
                 for (int m = 0; m < 32; ++m) {
                     const int i = 4 + (m >> 3), j = m & 7;
-                    acc[i][j] = mfma_16x16x128<BF, AF>(pack8(fb[P][j][0], fb[P][j][1]), pack8(fa[i % 5][0], fa[i % 5][1]), acc[i][j]);
+                    acc[i][j] = mfma_16x16x128<BF, AF>(pack8(fb[P][j][0], fb[P][j][1]), pack8(fa[(i - 1) % 5][0], fa[(i - 1) % 5][1]), acc[i][j]);
                     // a 16x16x128 MFMA lasts 32 clocks: room for about one memory instruction
                     // beside it.  Even slots take the 16 loads of the K tile after next, odd
-                    // slots the 16 reads of the next B fragments, slots 28 and 30 also the
-                    // two reads of the next first A fragment.
+                    // slots the 16 reads of the next B fragments, slots 0 and 2 also the two
+                    // reads of the next first A fragment (its own registers: free since block row 0).
                     if ((m & 1) == 0) {
                         if (load && (m >> 1) < S::LOADS) issue_load(m >> 1, t + 2, stage);
-                        if (next && m >= 28) read_a(0, (m >> 1) & 1, nstage);
+                        if (next && m < 4) read_a(0, (m >> 1) & 1, nstage);
                     } else if (next) {
                         read_b(PN{}, m >> 2, (m >> 1) & 1, nstage);
                     }

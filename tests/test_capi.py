@@ -68,7 +68,8 @@ def test_kernel_selection_is_pure_host_logic(pkg):
     s = L.fp8gemm_scratch_bytes(16, 28672, 8192)
     assert s % (16 * 8192 * 4) == 0        # whole partial-sum planes, or none
     # the plan behind the automatic selection: family, variant, K slices, columns | rotation
-    assert pkg.plan(8192, 8192, 8192) == (pkg.ALGO_TILE, 0, 1, 2)          # 256x256 persistent tiles, no slices
+    assert pkg.plan(8192, 8192, 8192) == (pkg.ALGO_TILE, 13, 1, 2)         # 256x256 persistent tiles on the 16x16x128 MFMA, no slices
+    assert pkg.plan(8192, 8320, 8192) == (pkg.ALGO_TILE, 0, 1, 2)          # odd count of 128-byte K tiles: the 32x32x64 form
     assert pkg.plan(8192, 8192, 8192, stages=4)[:3] == (pkg.ALGO_TILE, 1, 1)
     fam, var, slices, cols = pkg.plan(16, 8192, 28672)
     assert (fam, slices, cols) == (pkg.ALGO_SKINNY, 1, 64)
