@@ -273,11 +273,11 @@ hipError_t launch_ptile_shape(int m, int k, int n, const uint8_t *a, const uint8
     return hipErrorInvalidValue;
 }
 
-// The 16x16x128 form of the 256 x 256 tile walks K in pairs of 128-byte K tiles: every work
-// item (a tile, or one of its nsplit K slices) must hold an even number of them.
+// The 16x16x128 form of the 256 x 256 tile needs whole 128-byte K tiles, at least two per
+// work item (a tile, or one of its nsplit K slices).
 bool p2h_ok(int k, int nsplit)
 {
-    return k % 128 == 0 && (k / 128) % (2 * nsplit) == 0;
+    return k % 128 == 0 && (k / 128) / nsplit >= 2;
 }
 
 template <int AF, int BF>
@@ -421,7 +421,7 @@ struct TilePlan {
 };
 
 // Cost model behind the choice, in microseconds, fitted to MI355X timings of the
-// persistent kernels (128-byte K tiles; 45 shapes x 5 tile shapes x 12 ways of cutting K;
+// persistent kernels (128-byte K tiles; 45 shapes x 6 tile kernels x 12 ways of cutting K;
 // the pick is within 1 % of the best measured candidate on average):
 //   a round of 256 whole tiles     = k_tiles * per_k_tile + per_item
 //   a round of tail items          = k_tiles_per_slice * per_k_tile * load + per_item
@@ -435,11 +435,13 @@ struct PtileCost {
     double per_k_tile, per_item, stream_rate;   // us, us, bytes per us
 };
 constexpr PtileCost kPtileCosts[] = {
-    {0, 1, 256, 256, 1.40, 13.0, 4.0e6},
-    {9, 10, 192, 256, 1.25, 11.0, 4.6e6},
+    {0, 1, 256, 256, 1.30, 13.0, 4.0e6},
+    {13, -1, 256, 256, 1.25, 13.0, 4.0e6},     // the same tile on the 16x16x128 MFMA: less energy per flop, and
+                                               // the compute-bound shapes run at the board's power limit
+    {9, 10, 192, 256, 1.15, 9.0, 3.4e6},
     {5, 11, 128, 256, 1.00, 8.0, 5.0e6},
-    {6, 12, 128, 128, 0.75, 4.5, 3.2e6},
-    {8, -1, 256, 128, 0.90, 10.0, 4.0e6},
+    {6, 12, 128, 128, 0.75, 2.5, 3.2e6},
+    {8, -1, 256, 128, 0.90, 8.0, 4.6e6},
 };
 constexpr double kIdleChipFactor = 0.5;
 constexpr int kSplitChoices[] = {1, 2, 3, 4, 6, 8, 12, 16};
@@ -470,6 +472,7 @@ TilePlan plan_tile(int m, int k, int n, int stages)
                 if (split > 1 && (w.nsplit == 1 || kt / split < kMinKTilesPerSlice ||
                                   ptile_scratch_bytes(w, c.bm, c.bn) > kMaxSplitScratch))
                     continue;
+                if (c.variant == 13 && !p2h_ok(k, w.nsplit)) continue;
                 // whole-tile rounds run with every CU busy; the rounds of tail items with
                 // whatever share of the CUs they fill
                 double cost = (w.bulk / 256) * (kt * c.per_k_tile + c.per_item);
@@ -494,10 +497,6 @@ TilePlan plan_tile(int m, int k, int n, int stages)
     // K-walk rotation: per tile column while A is small enough to stay in an XCD's L2
     // next to the B rows in flight, else per XCD and round
     best.rotate = ((size_t)m * k <= ((size_t)2 << 20)) ? 1 : 2;
-    // the 256 x 256 tile runs on the 16x16x128 MFMA where its K walk allows it: the same
-    // tile, work list and traffic, about 8 % less energy per flop -- and the 8192^3-class
-    // shapes run at the board's power limit
-    if (best.variant == 0 && p2h_ok(k, best.nsplit)) best.variant = 13;
     return best;
 }
 
@@ -505,7 +504,7 @@ size_t tile_plan_scratch_bytes(int m, int n, const TilePlan &p)
 {
     if (p.nsplit <= 1) return 0;
     for (const PtileCost &c : kPtileCosts)
-        if (c.variant == p.variant || c.variant4 == p.variant || (c.variant == 0 && p.variant == 13)) {
+        if (c.variant == p.variant || c.variant4 == p.variant) {
             const PtileWork w = ptile_work(m, n, c.bm, c.bn, p.nsplit, p.split_all);
             return w.ok ? ptile_scratch_bytes(w, c.bm, c.bn) : 0;
         }

@@ -426,8 +426,6 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
             wait_vmcnt<0>();
             __syncthreads();
             if (1 < T) issue_all_loads(1, 1);
-#pragma unroll
-            for (int q = 0; q < 16; ++q) read_b(I0{}, q >> 1, q & 1, 0);
             read_a(0, 0, 0);
             read_a(0, 1, 0);
 
@@ -468,11 +466,21 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                 }
             };
             static_assert(S::LOADS <= 16, "the loads of a K tile are issued beside every other MFMA of block rows 4..7");
-            // T is even here (the host sends other K-tile counts to the 32x32x64 kernel): K tiles
-            // go in pairs, one per B fragment set, and the last pair is written out so that no
-            // branch surrounds a K tile (all 256 accumulation registers are taken; a copy of an
-            // accumulator at a join would have nowhere to go)
+            // K tiles go in pairs, one per B fragment set; an odd count starts with a single K
+            // tile on set 1.  T >= 2 (the host sends shorter K walks to the 32x32x64 kernel),
+            // so the last pair is written out and no branch surrounds a K tile inside the
+            // loop: all 256 accumulation registers are taken, and a copy of an accumulator
+            // at a join would have nowhere to go.
             int t = 0;
+            if (T & 1) {
+#pragma unroll
+                for (int q = 0; q < 16; ++q) read_b(I1{}, q >> 1, q & 1, 0);
+                ktile(I1{}, true, true, 0);
+                t = 1;
+            } else {
+#pragma unroll
+                for (int q = 0; q < 16; ++q) read_b(I0{}, q >> 1, q & 1, 0);
+            }
             for (; t < T - 2; t += 2) {
                 ktile(I0{}, true, true, t);
                 ktile(I1{}, true, true, t + 1);

@@ -69,21 +69,21 @@ def test_kernel_selection_is_pure_host_logic(pkg):
     assert s % (16 * 8192 * 4) == 0        # whole partial-sum planes, or none
     # the plan behind the automatic selection: family, variant, K slices, columns | rotation
     assert pkg.plan(8192, 8192, 8192) == (pkg.ALGO_TILE, 13, 1, 2)         # 256x256 persistent tiles on the 16x16x128 MFMA, no slices
-    assert pkg.plan(8192, 8320, 8192) == (pkg.ALGO_TILE, 0, 1, 2)          # odd count of 128-byte K tiles: the 32x32x64 form
+    assert pkg.plan(8192, 8256, 8192) == (pkg.ALGO_TILE, 0, 1, 2)          # K not a multiple of 128: the 32x32x64 form
     assert pkg.plan(8192, 8192, 8192, stages=4)[:3] == (pkg.ALGO_TILE, 1, 1)
     fam, var, slices, cols = pkg.plan(16, 8192, 28672)
     assert (fam, slices, cols) == (pkg.ALGO_SKINNY, 1, 64)
     fam, var, slices, _ = pkg.plan(256, 28672, 8192)
     assert fam == pkg.ALGO_TILE and slices > 1
     assert pkg.plan(100, 100, 100)[0] == pkg.ALGO_DIRECT
-    for shape in [(256, 28672, 8192), (64, 28672, 8192), (300, 4096, 500), (8192, 8192, 8192), (4352, 4352, 4352)]:
+    for shape in [(256, 28672, 8192), (64, 28672, 8192), (300, 4096, 500), (8192, 8192, 8192), (7168, 7168, 7168)]:
         slices = pkg.plan(*shape)[2]
         assert (L.fp8gemm_scratch_bytes(*shape) > 0) == (slices > 1)
     assert L.fp8gemm_scratch_bytes(64, 28672, 8192) == pkg.plan(64, 28672, 8192)[2] * 64 * 8192 * 4
-    # 17 x 17 tiles of 256 x 256: one round of whole tiles, the 33 left over cut into K slices
-    fam, var, slices, mode = pkg.plan(4352, 4352, 4352)
+    # 28 x 28 tiles of 256 x 256: three rounds of whole tiles, the 16 left over cut into K slices
+    fam, var, slices, mode = pkg.plan(7168, 7168, 7168)
     assert fam == pkg.ALGO_TILE and slices > 1 and mode >= 16
-    assert L.fp8gemm_scratch_bytes(4352, 4352, 4352) == slices * 33 * 256 * 256 * 4
+    assert L.fp8gemm_scratch_bytes(7168, 7168, 7168) == slices * 16 * 256 * 256 * 4
     out = (ctypes.c_int * 4)()
     assert L.fp8gemm_plan(0, 1, 1, 2, out) == 1 and L.fp8gemm_plan(1, 1, 1, 3, out) == 1
     # few tiles and a long K: the tiled kernels cut K into slices, whole planes of partial sums
