@@ -25,7 +25,7 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E peak, GB/s
 # HBM bytes moved by one 8192^3 launch of the tiled kernel, from rocprofv3
 # FETCH_SIZE / WRITE_SIZE counter runs scaled by the reading of a plain copy
 # kernel of known size (summary under profiles/).
-TRAFFIC_BYTES_8192 = (2 * 393683 + 262486) * 1024   # FETCH_SIZE x 2.0 (copy-kernel scale) + WRITE_SIZE x 1.0, KiB -> bytes
+TRAFFIC_BYTES_8192 = (2 * 393411 + 262872) * 1024   # FETCH_SIZE x 2.0 (copy-kernel scale) + WRITE_SIZE x 1.0, KiB -> bytes
 
 
 def load_package():
