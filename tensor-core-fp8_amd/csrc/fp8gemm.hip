@@ -436,8 +436,11 @@ struct PtileCost {
 };
 constexpr PtileCost kPtileCosts[] = {
     {0, 1, 256, 256, 1.30, 13.0, 4.0e6},
-    {13, -1, 256, 256, 1.25, 13.0, 4.0e6},     // the same tile on the 16x16x128 MFMA: less energy per flop, and
-                                               // the compute-bound shapes run at the board's power limit
+    {13, 13, 256, 256, 1.25, 13.0, 4.0e6},     // the same tile on the 16x16x128 MFMA: less energy per flop, and
+                                               // the compute-bound shapes run at the board's power limit.  One MFMA
+                                               // step takes 128 bytes of K, so a 4-deep ring of 64-byte K tiles and
+                                               // a 2-deep ring of 128-byte ones are the same pipeline: the 4-stage
+                                               // entry points share this kernel with the 2-stage ones
     {9, 10, 192, 256, 1.15, 9.0, 3.4e6},
     {5, 11, 128, 256, 1.00, 8.0, 5.0e6},
     {6, 12, 128, 128, 0.75, 2.5, 3.2e6},
