@@ -42,7 +42,11 @@ extern "C" {
  * (m, k, n, a, b, out) as there, default stream as there
  * (GEMM/src/gemm.cu:263-285).  "stage2" backs gemm::GEMM, "stage4" backs
  * gemm::GEMM4; the stage count selects the LDS pipeline depth of the tiled
- * kernel and never changes the result's contract.
+ * kernel (2- and 3-deep rings of 128-byte K tiles, or 4-deep rings of 64-byte
+ * ones) and never changes the result's contract.  Where the planned kernel
+ * computes with the 16x16x128 MFMA, one MFMA step consumes 128 bytes of K, a
+ * 4-deep ring of 64-byte K tiles and a 2-deep ring of 128-byte ones are the
+ * same pipeline, and both stage counts run the same kernel.
  */
 int fp8gemm_e4m3_e4m3_stage2(int m, int k, int n, const void *a, const void *b, float *out); /* gemm.cuh:12-15 */
 int fp8gemm_e4m3_e4m3_stage4(int m, int k, int n, const void *a, const void *b, float *out); /* gemm.cuh:18-21 */
