@@ -26,6 +26,7 @@ constexpr int kMaxDevices = 64;
 // Tiled kernel shapes: <BM, BN, BK, waves_m, waves_n, stages, swizzle>.
 using TileP2 = TileShape<256, 256, 128, 2, 2, 2, 3>;  // persistent, 2 x 64 KiB ring, 128x128 per wave
 using TileP2h = TileShape<256, 256, 128, 2, 2, 2, 3, true>;   // the same on v_mfma_f32_16x16x128_f8f6f4
+using TileT2h = TileShape<192, 256, 128, 2, 2, 2, 3, true>;   // 192 x 256 on that MFMA
 using TileP4 = TileShape<256, 256, 64, 2, 2, 4, 2>;   // persistent, 4 x 32 KiB ring
 using TileP8 = TileShape<256, 256, 128, 2, 4, 2, 3>;  // persistent, 8 waves, 128x64 per wave
 using TileS2 = TileShape<128, 128, 128, 2, 2, 2, 3>;  // one tile per workgroup, for small problems
@@ -39,7 +40,7 @@ using TileT2 = TileShape<192, 256, 128, 2, 2, 2, 3>;  // persistent, three-quart
 using TileT4 = TileShape<192, 256, 64, 2, 2, 4, 2>;
 using TileH4 = TileShape<128, 256, 64, 2, 2, 4, 2>;
 using TileQ4 = TileShape<128, 128, 64, 2, 2, 4, 2>;
-constexpr int kNumTileVariants = 14;              // 0 P2, 1 P4, 2 P8, 3 S2, 4 S4, 5 H3, 6 Q2, 7 S64, 8 W3, 9 T2, 10 T4, 11 H4, 12 Q4, 13 P2h
+constexpr int kNumTileVariants = 15;              // 0 P2, 1 P4, 2 P8, 3 S2, 4 S4, 5 H3, 6 Q2, 7 S64, 8 W3, 9 T2, 10 T4, 11 H4, 12 Q4, 13 P2h, 14 T2h
 
 // Skinny kernel shapes: <MT, TN, BK, stages>.
 template <int MT, int TN>
@@ -273,7 +274,7 @@ hipError_t launch_ptile_shape(int m, int k, int n, const uint8_t *a, const uint8
     return hipErrorInvalidValue;
 }
 
-// The 16x16x128 form of the 256 x 256 tile needs whole 128-byte K tiles, at least two per
+// The 16x16x128 forms of the 256 x 256 and 192 x 256 tiles need whole 128-byte K tiles, at least two per
 // work item (a tile, or one of its nsplit K slices).
 bool p2h_ok(int k, int nsplit)
 {
@@ -305,6 +306,9 @@ hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, 
     case 13:
         if (!p2h_ok(k, nsplit)) return hipErrorInvalidValue;
         return launch_ptile_shape<TileP2h, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
+    case 14:
+        if (!p2h_ok(k, nsplit)) return hipErrorInvalidValue;
+        return launch_ptile_shape<TileT2h, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -442,6 +446,7 @@ constexpr PtileCost kPtileCosts[] = {
                                                // a 2-deep ring of 128-byte ones are the same pipeline: the 4-stage
                                                // entry points share this kernel with the 2-stage ones
     {9, 10, 192, 256, 1.15, 9.0, 3.4e6},
+    {14, 14, 192, 256, 1.06, 9.0, 3.4e6},
     {5, 11, 128, 256, 1.00, 8.0, 5.0e6},
     {6, 12, 128, 128, 0.75, 2.5, 3.2e6},
     {8, -1, 256, 128, 0.90, 8.0, 4.6e6},
@@ -475,7 +480,7 @@ TilePlan plan_tile(int m, int k, int n, int stages)
                 if (split > 1 && (w.nsplit == 1 || kt / split < kMinKTilesPerSlice ||
                                   ptile_scratch_bytes(w, c.bm, c.bn) > kMaxSplitScratch))
                     continue;
-                if (c.variant == 13 && !p2h_ok(k, w.nsplit)) continue;
+                if ((c.variant == 13 || c.variant == 14) && !p2h_ok(k, w.nsplit)) continue;
                 // whole-tile rounds run with every CU busy; the rounds of tail items with
                 // whatever share of the CUs they fill
                 double cost = (w.bulk / 256) * (kt * c.per_k_tile + c.per_item);

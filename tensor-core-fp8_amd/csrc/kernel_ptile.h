@@ -401,13 +401,18 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
             // ---- v_mfma_f32_16x16x128_f8f6f4: one MFMA K step per K tile -------------
             // Lane (hi = lane % 16, hq = lane / 16) feeds row hi of a 16-row block with K
             // quarter hq (chunks 2*hq, 2*hq + 1 of the row).  The B fragments of a K tile
-            // (8 blocks, 64 registers) stay resident for its 64 MFMAs and are double
-            // buffered across K tiles; the A fragments stream through: blocks 1..7 are read
-            // during block rows 0..3 (two reads in every four MFMAs), so that every read of the
-            // ring slot has been issued by the middle of the K tile.  There the one barrier of the K tile sits: the next K
-            // tile has landed (its B fragments and first A fragment are read during block rows
-            // 4..7) and the slot just read is free for the K tile after that.
-            static_assert(STAGES == 2 && KSTEPS == 2 && TM == 4 && TN == 4, "the 16x16x128 schedule is written for 128 x 128 per wave, 128-byte K tiles, two ring slots");
+            // (8 blocks, 64 registers) stay resident for all its MFMAs and are double
+            // buffered across K tiles; the A fragments (8 blocks for 128 rows per wave, 6 for
+            // 96) stream through: all but the first are read during the first FIRST MFMAs, so
+            // that every read of the ring slot has been issued when the one barrier of the K
+            // tile comes, 32 MFMAs before its end.  By then the next K tile has landed (its B
+            // fragments and first A fragment are read during those last 32 MFMAs) and the slot
+            // just read is free for the K tile after that.
+            static_assert(STAGES == 2 && KSTEPS == 2 && (TM == 4 || TM == 3) && TN == 4,
+                          "the 16x16x128 schedule is written for 128 or 96 x 128 per wave, 128-byte K tiles, two ring slots");
+            constexpr int ABLK = 2 * TM;                  // A blocks of 16 rows per wave
+            constexpr int FIRST = 8 * ABLK - 32;          // MFMAs before the barrier
+            constexpr int ASTEP = FIRST / (ABLK - 1);     // A block b is read beside MFMAs ASTEP*(b-1), +1
             const int hi = lane & 15, hq = lane >> 4;
             const int hsw = tile_swizzle<BK, S::SWZ>(hi);             // same for rows hi + 16 * block
             const uint32_t hoff0 = (uint32_t)(((2 * hq) ^ hsw) * 16), hoff1 = (uint32_t)(((2 * hq + 1) ^ hsw) * 16);
@@ -436,11 +441,11 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                 using PN = std::integral_constant<int, P ^ 1>;
                 const int stage = t & 1, nstage = stage ^ 1;
 #pragma unroll
-                for (int m = 0; m < 32; ++m) {
+                for (int m = 0; m < FIRST; ++m) {
                     const int i = m >> 3, j = m & 7;
                     acc[i][j] = mfma_16x16x128<BF, AF>(pack8(fb[P][j][0], fb[P][j][1]), pack8(fa[i == 0 ? 5 : (i - 1) % 5][0], fa[i == 0 ? 5 : (i - 1) % 5][1]), acc[i][j]);
                     // block b > 5 goes to the place of block b - 5, whose block row is over by then
-                    if (m < 28 && (m & 3) < 2) read_a(1 + (m >> 2), m & 1, stage);
+                    if (1 + m / ASTEP < ABLK && m % ASTEP < 2) read_a(1 + m / ASTEP, m % ASTEP, stage);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 if (next) {
@@ -450,10 +455,10 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                 }
 #pragma unroll
                 for (int m = 0; m < 32; ++m) {
-                    const int i = 4 + (m >> 3), j = m & 7;
+                    const int i = FIRST / 8 + (m >> 3), j = m & 7;
                     acc[i][j] = mfma_16x16x128<BF, AF>(pack8(fb[P][j][0], fb[P][j][1]), pack8(fa[(i - 1) % 5][0], fa[(i - 1) % 5][1]), acc[i][j]);
                     // a 16x16x128 MFMA lasts 32 clocks: room for about one memory instruction
-                    // beside it.  Even slots take the 16 loads of the K tile after next, odd
+                    // beside it.  Even slots take the loads (16 or 14) of the K tile after next, odd
                     // slots the 16 reads of the next B fragments, slots 0 and 2 also the two
                     // reads of the next first A fragment (its own registers: free since block row 0).
                     if ((m & 1) == 0) {
@@ -465,7 +470,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                     __builtin_amdgcn_sched_barrier(0);
                 }
             };
-            static_assert(S::LOADS <= 16, "the loads of a K tile are issued beside every other MFMA of block rows 4..7");
+            static_assert(S::LOADS <= 16, "the loads of a K tile are issued beside every other one of the last 32 MFMAs");
             // K tiles go in pairs, one per B fragment set; an odd count starts with a single K
             // tile on set 1.  T >= 2 (the host sends shorter K walks to the 32x32x64 kernel),
             // so the last pair is written out and no branch surrounds a K tile inside the

@@ -124,36 +124,38 @@ def test_every_tile_variant(pkg, oracle, variant, shape):
 @pytest.mark.parametrize("shape", [(256, 256, 256), (300, 512, 200), (1000, 1024, 900), (513, 768, 257), (64, 256, 2048),
                                    (768, 2048, 1280), (300, 384, 300), (512, 1152, 256), (256, 640, 512)])
 @pytest.mark.parametrize("fa,fb", PAIRS)
-def test_tile_variant_on_16x16x128_mfma(pkg, oracle, fa, fb, shape):
-    """The 256 x 256 persistent tile computed with v_mfma_f32_16x16x128_f8f6f4 (variant 13; K a
-    multiple of 128, odd and even counts of K tiles), all four pairings, on shapes that overhang
-    the tile in m and n."""
+@pytest.mark.parametrize("variant", [13, 14])
+def test_tile_variant_on_16x16x128_mfma(pkg, oracle, variant, fa, fb, shape):
+    """The 256 x 256 and 192 x 256 persistent tiles computed with v_mfma_f32_16x16x128_f8f6f4
+    (variants 13, 14; K a multiple of 128, odd and even counts of K tiles), all four pairings,
+    on shapes that overhang the tile in m and n."""
     M, K, N = shape
-    rng = np.random.default_rng(zlib.crc32(repr((13, fa, fb, shape)).encode()))
+    rng = np.random.default_rng(zlib.crc32(repr((variant, fa, fb, shape)).encode()))
     A = random_codes(rng, (M, K), fa)
     B = random_codes(rng, (N, K), fb)
     if fa == 1:
         A = np.where(((A >> 2) & 0x1F) > 24, A & 0x83 | 0x3C, A).astype(np.uint8)
     if fb == 1:
         B = np.where(((B >> 2) & 0x1F) > 24, B & 0x83 | 0x3C, B).astype(np.uint8)
-    C = run_gpu(pkg, A, fa, B, fb, algo=ALGOS["tile"], variant=13)
+    C = run_gpu(pkg, A, fa, B, fb, algo=ALGOS["tile"], variant=variant)
     assert_within_bound(oracle, C, A, fa, B, fb, hw_term=True, block=128)     # one MFMA spans 128 of K here
 
 
-def test_16x16x128_variant_refuses_a_single_k_tile(pkg):
+@pytest.mark.parametrize("variant", [13, 14])
+def test_16x16x128_variant_refuses_a_single_k_tile(pkg, variant):
     A = np.zeros((256, 128), np.uint8)
     B = np.zeros((256, 128), np.uint8)
     with pytest.raises(RuntimeError):
-        run_gpu(pkg, A, 0, B, 0, algo=ALGOS["tile"], variant=13)
+        run_gpu(pkg, A, 0, B, 0, algo=ALGOS["tile"], variant=variant)
 
 
-@pytest.mark.parametrize("variant,split", [(0, 2), (0, 3), (1, 5), (5, 4), (5, 7), (6, 2), (6, 16), (2, 2), (8, 3), (13, 2), (13, 4)])
+@pytest.mark.parametrize("variant,split", [(0, 2), (0, 3), (1, 5), (5, 4), (5, 7), (6, 2), (6, 16), (2, 2), (8, 3), (13, 2), (13, 4), (14, 3)])
 @pytest.mark.parametrize("shape", [(256, 2048, 512), (300, 4096, 200), (1000, 2304, 900), (128, 8192, 2048)])
 def test_tile_k_slices(pkg, oracle, variant, split, shape):
     """Persistent tiled kernels with the K range cut into slices whose partial sums are
     added by the reduction kernel (uneven slices included), on shapes that overhang the tile."""
     M, K, N = shape
-    if variant == 13 and (K // 128) // split < 2:
+    if variant in (13, 14) and (K // 128) // split < 2:
         pytest.skip("the 16x16x128 variant takes at least two 128-byte K tiles per slice")
     A = pkg.fill((M, K), 1, seed=0xA11CE + K + split, dist="normal", sigma=4.0)
     B = pkg.fill((N, K), 0, seed=0xB0B + K + split, dist="normal", sigma=4.0)
