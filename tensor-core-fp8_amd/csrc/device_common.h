@@ -44,6 +44,28 @@ __device__ __forceinline__ v8i pack8(v4i lo, v4i hi)
     return r;
 }
 
+// Numbering of the tiles of C, shared by the persistent kernel and the reduction of its K
+// slices: column blocks of CB tile columns (CB >= tiles_n: a single block), inside a block
+// strips of GM tile rows, inside a strip down a column first.  256 consecutive numbers are
+// then a compact window of (256 / CB) x CB tiles where the matrix is large enough, and 32
+// consecutive ones a window of GM x (32 / GM).
+__device__ __forceinline__ void tile_of_number(int g, int tiles_m, int tiles_n, int GM, int CB, int &tm, int &tn)
+{
+    const int block_tiles = tiles_m * CB;
+    const int cb = g / block_tiles;
+    const int gb = g - cb * block_tiles;
+    int w = tiles_n - cb * CB;
+    w = w > CB ? CB : w;
+    const int per_strip = GM * w;
+    const int strip = gb / per_strip;
+    const int rem = gb - strip * per_strip;
+    int h = tiles_m - strip * GM;
+    h = h > GM ? GM : h;
+    const int col = rem / h;
+    tn = cb * CB + col;
+    tm = strip * GM + rem - col * h;
+}
+
 // What a kernel does with a finished fp32 sum: multiply by alpha * a_scale * b_scale and
 // store as fp32, bf16 or fp16 (round to nearest even).  The scale pointers are device
 // pointers to one float each, or null for 1.  The plain entry points use {1, null, null,

@@ -101,7 +101,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                                                                  const uint8_t *__restrict__ B,
                                                                  void *__restrict__ C,
                                                                  float *__restrict__ ws,
-                                                                 int tiles_m, int tiles_n, int GM,
+                                                                 int tiles_m, int tiles_n, int GM, int CB,
                                                                  int bulk, int tail, int nsplit,
                                                                  int rounds, int rotate, OutSpec spec)
 {
@@ -135,7 +135,9 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
 
     // Work items.  The tiles of C are numbered along strips of GM tile rows (down a
     // column of the strip first, then on to the next column), so that consecutive tile
-    // numbers form compact GM-row windows.  The first `bulk` tiles (a multiple of 256)
+    // numbers form compact GM-row windows; where B is too large for the last-level cache
+    // the strips are cut into blocks of CB columns, so that a round of 256 tiles covers a
+    // square window and reads far fewer rows of B.  The first `bulk` tiles (a multiple of 256)
     // are items of their own, 256 per round: XCD x takes 32 consecutive ones, one per
     // CU, and shares their operand panels in its L2 (workgroups with equal id mod 8 sit
     // on one XCD).  The last `tail` tiles, too few to fill a round, are cut into nsplit
@@ -172,15 +174,11 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
             g = bulk + t;
             if (nsplit > 1) ws_slot = slice * tail + t;
         }
-        const int per_strip = GM * tiles_n;
-        const int strip = g / per_strip;
-        const int rem = g - strip * per_strip;
-        int h = tiles_m - strip * GM;
-        h = h > GM ? GM : h;
-        const int col = rem / h;
+        int row, col;
+        tile_of_number(g, tiles_m, tiles_n, GM, CB, row, col);
         // (the divisions may run on the vector unit; every lane holds the same values)
         tn = __builtin_amdgcn_readfirstlane(col);
-        tm = __builtin_amdgcn_readfirstlane(strip * GM + rem - col * h);
+        tm = __builtin_amdgcn_readfirstlane(row);
         const int split = r < bulk_rounds ? 1 : nsplit;
         const int k0 = (int)((long)KT * slice / split);
         kt0 = __builtin_amdgcn_readfirstlane(k0);

@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce4_kernel(const v4f *__r
 __global__ __launch_bounds__(256) void gemm_tile_slices_reduce_kernel(const float *__restrict__ ws,
                                                                       void *__restrict__ C, int M, int N,
                                                                       int BM, int BN, int tiles_m, int tiles_n,
-                                                                      int GM, int bulk, int tail, int nsplit,
+                                                                      int GM, int CB, int bulk, int tail, int nsplit,
                                                                       OutSpec spec)
 {
     const int quads_per_tile = BM * BN / 4;
@@ -59,13 +59,8 @@ __global__ __launch_bounds__(256) void gemm_tile_slices_reduce_kernel(const floa
     const int row = q / (BN / 4);
     const int col = (q - row * (BN / 4)) * 4;
     const int g = bulk + u;
-    const int per_strip = GM * tiles_n;
-    const int strip = g / per_strip;
-    const int rem = g - strip * per_strip;
-    int h = tiles_m - strip * GM;
-    h = h > GM ? GM : h;
-    const int tn = rem / h;
-    const int tm = strip * GM + rem - tn * h;
+    int tm, tn;
+    tile_of_number(g, tiles_m, tiles_n, GM, CB, tm, tn);
     const int grow = tm * BM + row;
     const int gcol = tn * BN + col;
     if (grow >= M || gcol >= N) return;

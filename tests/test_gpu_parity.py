@@ -306,6 +306,25 @@ def test_stage4_entry_follows_the_same_plans(pkg, oracle, shape):
     assert worst < 0.5
 
 
+@pytest.mark.parametrize("variant,split", [(13, -2), (0, 0), (14, 0)])
+def test_column_blocked_tile_numbering(pkg, oracle, variant, split):
+    """B of 192 MiB and more beside a smaller A: the tiles are numbered in blocks of 16 tile columns (whole rounds,
+    leftover tiles cut into K slices and their reduction all use that numbering).  Sampled rows
+    against the oracle, every tile row and every column covered."""
+    M, K, N = 4352, 12288, 16384
+    A = pkg.fill((M, K), 0, seed=0xC0FFEE, dist="normal", sigma=1.0)
+    B = pkg.fill((N, K), 0, seed=0xBEEF, dist="normal", sigma=1.0)
+    C = run_gpu(pkg, A, 0, B, 0, algo=ALGOS["tile"], variant=variant, split_k=split)
+    rows = np.arange(5, M, 251, dtype=np.int32)
+    worst = assert_within_bound(oracle, C, A, 0, B, 0, rows=rows)
+    assert worst < 0.25
+    # every row: the row sums of C against A times the column sums of B (exact in float64 up to the kernel's rounding)
+    bsum = oracle.decode(B, 0).astype(np.float64).sum(axis=0)
+    want = oracle.decode(A, 0).astype(np.float64) @ bsum
+    got = C.astype(np.float64).sum(axis=1)
+    assert np.abs(got - want).max() <= 1e-3 * np.abs(C).astype(np.float64).sum(axis=1).max()
+
+
 def test_scratch_grows_and_is_reused_across_calls_and_streams(pkg, oracle):
     """Calls that need the partial-sum scratch, in growing and shrinking order, on the default
     stream and on a side stream (ordered by the caller): every result is right, before and
