@@ -116,6 +116,15 @@ int fp8gemm_select_algo(int m, int k, int n);
  * Returns 0, or hipErrorInvalidValue for bad arguments. */
 int fp8gemm_plan(int m, int k, int n, int stages, int plan[4]);
 
+/*
+ * Order in which the persistent tiled kernel walks the bm x bn tiles of C for a
+ * shape (pure host logic, for tests): tile number `index` (0 .. tiles-1) ->
+ * its tile row and tile column.  256 consecutive numbers run at the same time,
+ * 32 consecutive ones on one XCD.  No counterpart in the reference, whose
+ * kernels take the tile from blockIdx (GEMM/src/gemm.cu:39-44).
+ */
+int fp8gemm_tile_order(int m, int k, int n, int bm, int bn, int index, int *tile_row, int *tile_col);
+
 /* Bytes of device scratch (partial sums of K slices) the library keeps cached
  * per device for a shape (0 when the shape needs none).  The scratch is the
  * only allocation the library ever makes; it is grown on demand, reused by

@@ -49,7 +49,7 @@ __device__ __forceinline__ v8i pack8(v4i lo, v4i hi)
 // strips of GM tile rows, inside a strip down a column first.  256 consecutive numbers are
 // then a compact window of (256 / CB) x CB tiles where the matrix is large enough, and 32
 // consecutive ones a window of GM x (32 / GM).
-__device__ __forceinline__ void tile_of_number(int g, int tiles_m, int tiles_n, int GM, int CB, int &tm, int &tn)
+__host__ __device__ __forceinline__ void tile_of_number(int g, int tiles_m, int tiles_n, int GM, int CB, int &tm, int &tn)
 {
     const int block_tiles = tiles_m * CB;
     const int cb = g / block_tiles;

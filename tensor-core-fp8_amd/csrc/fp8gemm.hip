@@ -683,6 +683,15 @@ int fp8gemm_plan(int m, int k, int n, int stages, int plan[4])
     return 0;
 }
 
+int fp8gemm_tile_order(int m, int k, int n, int bm, int bn, int index, int *tile_row, int *tile_col)
+{
+    if (m <= 0 || k <= 0 || n <= 0 || bm <= 0 || bn <= 0 || !tile_row || !tile_col) return (int)hipErrorInvalidValue;
+    const PtileWork w = ptile_work(m, n, bm, bn, 1, false);
+    if (!w.ok || index < 0 || index >= w.tiles_m * w.tiles_n) return (int)hipErrorInvalidValue;
+    tile_of_number(index, w.tiles_m, w.tiles_n, w.GM, tile_column_block(w.tiles_n, m, n, k), *tile_row, *tile_col);
+    return 0;
+}
+
 size_t fp8gemm_scratch_bytes(int m, int k, int n)
 {
     if (m <= 0 || k <= 0 || n <= 0) return 0;

@@ -128,3 +128,37 @@ def test_python_entry_points_refuse_host_tensors(pkg):
     a = torch.zeros((16, 128), dtype=torch.uint8)
     with pytest.raises(pkg.Fp8GemmError):
         pkg.gemm(a, a, a_fmt=0, b_fmt=0)
+
+
+def test_tile_order_is_a_bijection_with_compact_windows(pkg):
+    """The persistent kernel's tile numbering (host copy of the device function): every tile
+    exactly once, for plain strips and for the numbering in blocks of 16 tile columns; 32
+    consecutive numbers (one XCD) touch at most two strips of 4 tile rows."""
+    import ctypes
+    L = pkg.lib()
+    L.fp8gemm_tile_order.restype = ctypes.c_int
+    L.fp8gemm_tile_order.argtypes = [ctypes.c_int] * 6 + [ctypes.POINTER(ctypes.c_int)] * 2
+    tr, tc = ctypes.c_int(), ctypes.c_int()
+    cases = [((1000, 512, 900), 256, 256), ((4352, 4352, 4352), 256, 256), ((300, 1024, 5000), 128, 128),
+             ((4352, 12288, 16384), 256, 256),      # B of 192 MiB beside a smaller A: blocks of 16 tile columns
+             ((1100, 16384, 20000), 192, 256), ((256, 1024, 256), 256, 256)]
+    for (m, k, n), bm, bn in cases:
+        tm, tn = -(-m // bm), -(-n // bn)
+        seen = set()
+        order = []
+        for g in range(tm * tn):
+            assert L.fp8gemm_tile_order(m, k, n, bm, bn, g, ctypes.byref(tr), ctypes.byref(tc)) == 0
+            assert 0 <= tr.value < tm and 0 <= tc.value < tn
+            seen.add((tr.value, tc.value))
+            order.append((tr.value, tc.value))
+        assert len(seen) == tm * tn, (m, k, n)
+        for g0 in range(0, tm * tn - 31, 32):
+            rows = {r for r, _ in order[g0:g0 + 32]}
+            assert len(rows) <= 8, (m, k, n, g0)                  # at most two strips of 4 rows
+    assert L.fp8gemm_tile_order(256, 256, 256, 256, 256, 1, ctypes.byref(tr), ctypes.byref(tc)) != 0
+    # blocked numbering: the first 256 tiles of the 17 x 64 grid form a 16 x 16 window
+    first = [None] * 256
+    for g in range(256):
+        L.fp8gemm_tile_order(4352, 12288, 16384, 256, 256, g, ctypes.byref(tr), ctypes.byref(tc))
+        first[g] = (tr.value, tc.value)
+    assert {r for r, _ in first} == set(range(16)) and {c for _, c in first} == set(range(16))
