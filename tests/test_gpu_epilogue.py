@@ -41,6 +41,8 @@ SHAPES = [
     (256, 8192, 1024),      # tiled kernel with K slices + tile-slot reduction
     (70, 200, 90),          # general kernel (k not a multiple of 16)
     (512, 1040, 384),       # K tile overhanging K
+    (3584, 256, 3584),      # 256 x 256 tiles on the 16x16x128 MFMA
+    (3072, 384, 3072),      # 192 x 256 tiles on the 16x16x128 MFMA, odd count of K tiles
 ]
 
 
