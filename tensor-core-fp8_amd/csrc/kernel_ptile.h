@@ -18,6 +18,12 @@
 // instructions and the texture-address unit sees an even stream (four waves x
 // one 1 KiB load per MFMA slot is its full rate of 64 B/clk).
 //
+// Two forms of the K loop, chosen by the tile shape type: v_mfma_f32_32x32x64_f8f6f4 with
+// ping-pong fragment sets (above), and v_mfma_f32_16x16x128_f8f6f4 (S::MF16) with the B
+// fragments of a K tile resident and the A fragments streamed; the second needs less
+// energy per flop, which is what limits the large shapes on a power-capped board.  Loads,
+// ring, work list and epilogue are shared.
+//
 // MFMA operand roles are swapped (src0 = B rows, src1 = A rows): the result
 // registers of a lane are then 4 consecutive columns of one row of C, which
 // turns the epilogue into 128-bit stores.
@@ -94,7 +100,9 @@ __device__ __forceinline__ v4i make_buffer_resource(const void *base, unsigned l
 
 // KOVER: the last K tile may overhang K (K % BK != 0); compiled separately so that the
 // common case carries no test for it.  EX: the output goes through `spec` (scale, fp32 /
-// bf16 / fp16); without it C receives the bare fp32 sums and `spec` is ignored.
+// bf16 / fp16); without it C receives the bare fp32 sums and `spec` is ignored.  BSTREAM: B is
+// loaded with the non-temporal hint (for a C with a single row of tiles, where every byte of B
+// is read by exactly one workgroup).
 template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM>
 __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, int N,
                                                                  const uint8_t *__restrict__ A,
