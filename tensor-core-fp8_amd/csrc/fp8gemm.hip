@@ -441,11 +441,11 @@ struct TilePlan {
 };
 
 // Cost model behind the choice, in microseconds, fitted to MI355X timings of the
-// persistent kernels (128-byte K tiles; 45 shapes x 6 tile kernels x 12 ways of cutting K;
+// persistent kernels (128-byte K tiles; 45 shapes x 7 tile kernels x 12 ways of cutting K;
 // the pick is within 1 % of the best measured candidate on average):
 //   a round of 256 whole tiles     = k_tiles * per_k_tile + per_item
 //   a round of tail items          = k_tiles_per_slice * per_k_tile * load + per_item
-//   load                           = 0.5 + 0.5 * (share of the 256 CUs with an item): a chip
+//   load                           = 0.6 + 0.4 * (share of the 256 CUs with an item): a chip
 //                                    that is partly idle clocks higher and contends less
 //   main kernel                    = max(sum of rounds, input_bytes / stream_rate)
 //   K slices add one reduction pass over (nsplit + 1) x the cut tiles.
@@ -461,13 +461,13 @@ constexpr PtileCost kPtileCosts[] = {
                                                // step takes 128 bytes of K, so a 4-deep ring of 64-byte K tiles and
                                                // a 2-deep ring of 128-byte ones are the same pipeline: the 4-stage
                                                // entry points share this kernel with the 2-stage ones
-    {9, 10, 192, 256, 1.15, 9.0, 3.4e6},
-    {14, 14, 192, 256, 1.06, 9.0, 3.4e6},
-    {5, 11, 128, 256, 1.00, 8.0, 5.0e6},
-    {6, 12, 128, 128, 0.75, 2.5, 3.2e6},
-    {8, -1, 256, 128, 0.90, 8.0, 4.6e6},
+    {9, 10, 192, 256, 1.15, 9.0, 4.6e6},
+    {14, 14, 192, 256, 1.10, 9.0, 4.0e6},
+    {5, 11, 128, 256, 1.00, 6.0, 5.0e6},
+    {6, 12, 128, 128, 0.75, 2.5, 4.0e6},
+    {8, -1, 256, 128, 0.90, 10.0, 4.6e6},
 };
-constexpr double kIdleChipFactor = 0.5;
+constexpr double kIdleChipFactor = 0.6;
 constexpr int kSplitChoices[] = {1, 2, 3, 4, 6, 8, 12, 16};
 constexpr int kMinKTilesPerSlice = 12;
 constexpr size_t kMaxSplitScratch = (size_t)1 << 30;
@@ -509,7 +509,7 @@ TilePlan plan_tile(int m, int k, int n, int stages)
                 }
                 const double stream = ((double)m * k + (double)n * k) / c.stream_rate;
                 if (stream > cost) cost = stream;
-                if (w.nsplit > 1) cost += 4.0 + (w.nsplit + 1) * (double)w.tail * c.bm * c.bn * 4.0 / 6.0e6;
+                if (w.nsplit > 1) cost += 6.0 + (w.nsplit + 1) * (double)w.tail * c.bm * c.bn * 4.0 / 6.0e6;
                 if (cost < best_cost) {
                     best_cost = cost;
                     best.variant = stages == 4 ? c.variant4 : c.variant;
