@@ -463,7 +463,7 @@ constexpr PtileCost kPtileCosts[] = {
                                                // entry points share this kernel with the 2-stage ones
     {9, 10, 192, 256, 1.15, 9.0, 4.6e6},
     {14, 14, 192, 256, 1.10, 9.0, 4.0e6},
-    {5, 11, 128, 256, 1.00, 6.0, 5.0e6},
+    {5, 11, 128, 256, 1.00, 6.0, 6.5e6},
     {6, 12, 128, 128, 0.75, 2.5, 4.0e6},
     {8, -1, 256, 128, 0.90, 10.0, 4.6e6},
 };
