@@ -4,17 +4,28 @@
 One "step" is one launch of the hot path (a whole GEMM) through the C ABI on
 synthetic operands that are already resident in HBM.  The headline workload is
 the compute-bound square shape M=N=K=8192, e4m3 x e4m3 -> fp32; the same run
-also times the HBM-bound skinny shape M=16, N=28672, K=8192 and a bounded
-sample of the reference's CPU GEMM loop on the host cores.
+also times the LLM-linear skinny shapes (HBM-bound) and the reference's CPU
+GEMM loop on the host cores.
 
-Prints ONE JSON line (see the keys below).  `python bench.py --gpus N` with
-N > 1 exits with a message: this build measures one GPU.
+The 8192^3 kernel runs at the board's power limit, and the chip's power
+management takes some tens of milliseconds of continuous load to settle (the
+first launches after idle run at other clocks than the hundredth).  So that the
+timed steps show what a caller in a loop gets, whatever --warmup says, an
+untimed settle phase comes first: launches in blocks of 20 until three
+successive blocks agree within 2 % (at most 2 s).  The rate of the very first
+block after idle is reported beside it (`cold_burst`).
+
+Prints ONE JSON line.  `python bench.py --gpus N` with N > 1 exits with a
+message: this build measures one GPU.
 """
 import argparse
+import glob
 import importlib.util
 import json
 import os
+import statistics
 import sys
+import threading
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -22,10 +33,16 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 PEAK_FP8_TFLOPS = 5000.0     # MI355X dense FP8 MFMA peak, TFLOP/s
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E peak, GB/s
 
-# HBM bytes moved by one 8192^3 launch of the tiled kernel, from rocprofv3
-# FETCH_SIZE / WRITE_SIZE counter runs scaled by the reading of a plain copy
-# kernel of known size (summary under profiles/).
-TRAFFIC_BYTES_8192 = (2 * 393411 + 262872) * 1024   # FETCH_SIZE x 2.0 (copy-kernel scale) + WRITE_SIZE x 1.0, KiB -> bytes
+# HBM-side bytes moved by one 8192^3 launch of the tiled kernel: a constant taken from the
+# rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs summarised under profiles/ (each scaled by
+# what the same counter reads for a plain copy kernel of known size), not a reading of this run.
+TRAFFIC_8192 = {"fetch_kib": 393411, "fetch_scale": 2.0, "write_kib": 262872, "write_scale": 1.0}
+TRAFFIC_BYTES_8192 = int((TRAFFIC_8192["fetch_kib"] * TRAFFIC_8192["fetch_scale"] +
+                          TRAFFIC_8192["write_kib"] * TRAFFIC_8192["write_scale"]) * 1024)
+
+SETTLE_BLOCK = 20            # launches per settle block
+SETTLE_AGREE = 1.02          # three successive blocks within 2 %
+SETTLE_CAP_S = 2.0
 
 
 def load_package():
@@ -45,10 +62,89 @@ def load_oracle():
     return oracle
 
 
+class BoardSampler(threading.Thread):
+    """Shader clock and board power from sysfs while the timed launches run (both are
+    firmware averages; absent files are skipped)."""
+
+    def __init__(self):
+        super().__init__(daemon=True)
+        self.power_files = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input") + \
+            glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average")
+        self.cap_files = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap")
+        self.sclk_files = glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")
+        self.stop_flag = threading.Event()
+        self.power_w, self.sclk_mhz = [], []
+
+    @staticmethod
+    def _read(path):
+        try:
+            with open(path) as f:
+                return f.read()
+        except OSError:
+            return None
+
+    def run(self):
+        while not self.stop_flag.is_set():
+            for p in self.power_files[:1]:
+                v = self._read(p)
+                if v and v.strip().isdigit():
+                    self.power_w.append(int(v) / 1e6)
+            for p in self.sclk_files[:1]:
+                v = self._read(p) or ""
+                for line in v.splitlines():
+                    if line.rstrip().endswith("*"):
+                        digits = "".join(ch for ch in line.split(":")[1] if ch.isdigit())
+                        if digits:
+                            self.sclk_mhz.append(int(digits))
+            time.sleep(0.02)
+
+    def summary(self):
+        cap = None
+        for p in self.cap_files[:1]:
+            v = self._read(p)
+            if v and v.strip().isdigit():
+                cap = int(v) / 1e6
+        if not self.power_w and not self.sclk_mhz:
+            return {"available": False}
+        out = {"available": True, "samples": max(len(self.power_w), len(self.sclk_mhz)), "power_cap_w": cap}
+        if self.power_w:
+            out.update(power_w_last=self.power_w[-1], power_w_max=max(self.power_w))
+        if self.sclk_mhz:
+            out.update(shader_clock_mhz_last=self.sclk_mhz[-1], shader_clock_mhz_median=statistics.median(self.sclk_mhz),
+                       shader_clock_mhz_nominal=2400)
+        return out
+
+
+def time_block(torch, fn, n, offset=0):
+    """Milliseconds per launch over n back-to-back launches: HIP events on the launch stream."""
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(n):
+        fn(offset + i)
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / n
+
+
+def settle(torch, fn):
+    """Untimed: launches until the chip's clocks have settled under this load.  Returns the
+    per-launch time of every block (the first one is the burst right after idle)."""
+    blocks = [time_block(torch, fn, SETTLE_BLOCK)]
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < SETTLE_CAP_S:
+        blocks.append(time_block(torch, fn, SETTLE_BLOCK))
+        last = blocks[-3:]
+        if len(blocks) >= 4 and max(last) <= SETTLE_AGREE * min(last):
+            break
+    return blocks
+
+
 def time_launches(torch, fn, steps, warmup):
-    """Average milliseconds per launch: HIP events on the launch stream around `steps` launches."""
-    for _ in range(warmup):
-        fn(0)
+    """The contract's measurement: `warmup` untimed launches, then exactly `steps` timed ones
+    between synchronisations.  Returns (ms per launch by HIP events, by the host clock)."""
+    for i in range(warmup):
+        fn(i)
     torch.cuda.synchronize()
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
@@ -62,13 +158,17 @@ def time_launches(torch, fn, steps, warmup):
     return e0.elapsed_time(e1) / steps, wall_ms / steps
 
 
+LLM_SHAPES = [(n, k, m) for (n, k) in [(28672, 8192), (8192, 28672), (10240, 8192)] for m in (1, 16, 64, 256)]
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=300)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host CPU leg")
     ap.add_argument("--no-vendor", action="store_true", help="skip the hipBLASLt comparison (a child process)")
+    ap.add_argument("--no-llm-shapes", action="store_true", help="time only M=16 N=28672 K=8192 of the skinny shapes")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel that FETCH_SIZE / WRITE_SIZE "
                          "counter readings are scaled by when this script runs under rocprofv3 --pmc")
@@ -93,6 +193,19 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    L = pkg.lib()
+    stream = torch.cuda.current_stream().cuda_stream      # events and launches share this stream
+
+    def raw_launch(m, k, n, a, b, c):
+        """The bare C-ABI call (a few microseconds of host time, so short kernels stay back to back)."""
+        pa, pb, pc = a.data_ptr(), b.data_ptr(), c.data_ptr()
+
+        def go(_i):
+            code = L.fp8gemm_launch(m, k, n, pa, 0, pb, 0, pc, 2, stream)
+            if code != 0:
+                pkg.check(code)
+        return go
+
     # ---------------------------------------------------------------- square, compute-bound
     M = N = K = 8192
     A_h = pkg.fill((M, K), pkg.E4M3, seed=0xA11CE + 3, dist="normal")
@@ -100,22 +213,23 @@ def main():
     A = torch.from_numpy(A_h).to(dev)
     B = torch.from_numpy(B_h).to(dev)
     C = torch.empty((M, N), dtype=torch.float32, device=dev)
-    L = pkg.lib()
-    stream = torch.cuda.current_stream().cuda_stream      # events and launches share this stream
-
-    def raw_launch(m, k, n, a, b, c):
-        """The bare C-ABI call (a few microseconds of host time, so short kernels stay back to back)."""
-        pa, pb, pc = a.data_ptr(), b.data_ptr(), c.data_ptr()
-        def go(_i):
-            code = L.fp8gemm_launch(m, k, n, pa, 0, pb, 0, pc, 2, stream)
-            if code != 0:
-                pkg.check(code)
-        return go
-
-    ms, wall_ms = time_launches(torch, raw_launch(M, K, N, A, B, C), args.steps, args.warmup)
+    torch.cuda.synchronize()
     flops = 2.0 * M * N * K
-    tflops = flops / (ms * 1e-3) / 1e12
     alg_bytes = M * K + N * K + 4 * M * N
+
+    def to_tflops(ms):
+        return flops / (ms * 1e-3) / 1e12
+
+    go = raw_launch(M, K, N, A, B, C)
+    sampler = BoardSampler()
+    sampler.start()
+    settle_blocks = settle(torch, go)
+    ms, wall_ms = time_launches(torch, go, args.steps, args.warmup)
+    # the same measurement five more times, back to back: how far one block of `steps` launches scatters
+    repeat_ms = [time_block(torch, go, args.steps) for _ in range(5)]
+    sampler.stop_flag.set()
+    sampler.join()
+    tflops = to_tflops(ms)
 
     # parity on a sample of full rows, against the CPU oracle (checker only)
     parity = None
@@ -130,29 +244,51 @@ def main():
                   "pass": bool((err <= tol).all())}
     except Exception as ex:  # the oracle is only the checker; say so if it is unavailable
         parity = {"error": str(ex)[:200]}
+    del A, B, C
 
-    # ---------------------------------------------------------------- skinny, HBM-bound
-    m2, n2, k2 = 16, 28672, 8192
-    A2 = torch.from_numpy(pkg.fill((m2, k2), pkg.E4M3, seed=0xA11CE + 4, dist="normal")).to(dev)
-    W_h = pkg.fill((n2, k2), pkg.E4M3, seed=0xB0B + 4, dist="weights", sigma=0.02)
-    # six distinct weight buffers (1.4 GB): a launch finds nothing of its operand left in the
-    # 256 MB Infinity Cache (with three, about a tenth of B is still served from it)
-    NBUF = 6
-    Ws = [torch.from_numpy(W_h).to(dev)]
-    for j in range(1, NBUF):
-        Ws.append(Ws[0].clone())
-    C2 = torch.empty((m2, n2), dtype=torch.float32, device=dev)
-    gos = [raw_launch(m2, k2, n2, A2, W, C2) for W in Ws]
-    ms_cold, _ = time_launches(torch, lambda i: gos[i % NBUF](i), max(args.steps, 30), args.warmup)
-    ms_warm, _ = time_launches(torch, gos[0], max(args.steps, 30), args.warmup)
-    bytes2 = m2 * k2 + n2 * k2 + 4 * m2 * n2
+    # ---------------------------------------------------------------- LLM-linear shapes, HBM-bound
+    # Cold figures: every launch reads a weight buffer that has been pushed out of the 256 MB
+    # Infinity Cache by the launches before it (rotation over buffers totalling 1.2 GB and more).
+    def time_llm(n2, k2, ms_list, W_h):
+        res = []
+        nbuf = max(3, -(-(1200 << 20) // (n2 * k2)))
+        Ws = [torch.from_numpy(W_h).to(dev)]
+        for _ in range(1, nbuf):
+            Ws.append(Ws[0].clone())
+        for m2 in ms_list:
+            A2 = torch.from_numpy(pkg.fill((m2, k2), pkg.E4M3, seed=0xA11CE + 4 + m2, dist="normal")).to(dev)
+            C2 = torch.empty((m2, n2), dtype=torch.float32, device=dev)
+            gos = [raw_launch(m2, k2, n2, A2, W, C2) for W in Ws]
+            steps2 = max(args.steps, 60)
+            ms_cold, _ = time_launches(torch, lambda i: gos[i % nbuf](i), steps2, 30)
+            ms_warm, _ = time_launches(torch, gos[0], steps2, 30)
+            bytes2 = m2 * k2 + n2 * k2 + 4 * m2 * n2
+            flops2 = 2.0 * m2 * n2 * k2
+            gbs = bytes2 / (ms_cold * 1e-3) / 1e9
+            tf = flops2 / (ms_cold * 1e-3) / 1e12
+            res.append({"M": m2, "N": n2, "K": k2, "algorithmic_bytes": bytes2, "plan": list(pkg.plan(m2, k2, n2)),
+                        "us_cold": ms_cold * 1e3, "gbs_cold": gbs, "frac_hbm_peak_cold": gbs / PEAK_HBM_GBS,
+                        "tflops_cold": tf, "frac_fp8_peak_cold": tf / PEAK_FP8_TFLOPS,
+                        "us_warm": ms_warm * 1e3, "gbs_warm": bytes2 / (ms_warm * 1e-3) / 1e9,
+                        "weight_buffers": nbuf})
+        return res
+
+    llm = []
+    groups = [(28672, 8192, [16] if args.no_llm_shapes else [1, 16, 64, 256])]
+    if not args.no_llm_shapes:
+        groups += [(8192, 28672, [1, 16, 64, 256]), (10240, 8192, [1, 16, 64, 256])]
+    for gi, (n2, k2, ms_list) in enumerate(groups):
+        W_h = pkg.fill((n2, k2), pkg.E4M3, seed=0xB0B + 4 + gi, dist="weights", sigma=0.02)
+        llm += time_llm(n2, k2, ms_list, W_h)
+        torch.cuda.empty_cache()
+    head = [r for r in llm if (r["M"], r["N"], r["K"]) == (16, 28672, 8192)][0]
     skinny = {"workload": "M=16 N=28672 K=8192 e4m3 activations x e4m3 weights -> fp32",
-              "algorithmic_bytes": bytes2,
-              "us_cold": ms_cold * 1e3, "gbs_cold": bytes2 / (ms_cold * 1e-3) / 1e9,
-              "us_warm": ms_warm * 1e3, "gbs_warm": bytes2 / (ms_warm * 1e-3) / 1e9,
-              "frac_hbm_peak_cold": bytes2 / (ms_cold * 1e-3) / 1e9 / PEAK_HBM_GBS,
-              "note": "cold = rotating over 6 weight buffers (1.4 GB, nothing left in the 256 MB Infinity Cache), "
-                      "warm = same buffer every launch"}
+              "algorithmic_bytes": head["algorithmic_bytes"],
+              "us_cold": head["us_cold"], "gbs_cold": head["gbs_cold"],
+              "us_warm": head["us_warm"], "gbs_warm": head["gbs_warm"],
+              "frac_hbm_peak_cold": head["frac_hbm_peak_cold"],
+              "note": "cold = rotating over %d weight buffers (nothing of the next one left in the 256 MB Infinity "
+                      "Cache), warm = same buffer every launch" % head["weight_buffers"]}
 
     # ---------------------------------------------------------------- CPU baseline (host cores)
     cpu = None
@@ -162,19 +298,25 @@ def main():
             mc = nc = kc = 1024
             Ac = pkg.fill((mc, kc), pkg.E4M3, seed=0xA11CE + 1, dist="normal")
             Bc = pkg.fill((nc, kc), pkg.E4M3, seed=0xB0B + 1, dist="normal")
-            rows_c = 384                      # bounded sample: 384 of the 1024 rows, ~10 s single-thread
-            t0 = time.perf_counter()
-            oracle.gemm_verbatim(Ac[:rows_c], 0, Bc, 0)
-            t_verb = time.perf_counter() - t0
-            t0 = time.perf_counter()
-            oracle.gemm(Ac, 0, Bc, 0)
-            t_fast = time.perf_counter() - t0
-            cpu = {"value": 2.0 * rows_c * nc * kc / t_verb / 1e12, "unit": "TFLOPS", "cores": 1, "kind": "port",
-                   "sample": "first %d rows of the M=N=K=1024 e4m3 CPU-path configuration, the reference's m-n-k "
-                             "loop order, one thread, %.1f s" % (rows_c, t_verb),
-                   "all_cores": {"value": 2.0 * mc * nc * kc / t_fast / 1e12, "unit": "TFLOPS",
-                                 "cores": oracle.num_threads(),
-                                 "what": "bit-identical blocked/OpenMP form of the same loop, full 1024^3"}}
+            t_verb = []
+            for _ in range(3):
+                t0 = time.perf_counter()
+                oracle.gemm_verbatim(Ac, 0, Bc, 0)
+                t_verb.append(time.perf_counter() - t0)
+            t_fast = []
+            for _ in range(3):
+                t0 = time.perf_counter()
+                oracle.gemm(Ac, 0, Bc, 0)
+                t_fast.append(time.perf_counter() - t0)
+            fl = 2.0 * mc * nc * kc
+            cpu = {"value": fl / min(t_verb) / 1e12, "unit": "TFLOPS", "cores": 1, "kind": "port",
+                   "sample": "the whole M=N=K=1024 e4m3 CPU-path configuration, the reference's m-n-k loop order "
+                             "with one decode per operand per multiply, one thread, 3 repetitions "
+                             "(best %.2f s, mean %.2f s); value = best" % (min(t_verb), sum(t_verb) / 3),
+                   "seconds_best": min(t_verb), "seconds_mean": sum(t_verb) / 3, "host_cores": os.cpu_count(),
+                   "all_cores": {"value": fl / min(t_fast) / 1e12, "unit": "TFLOPS", "cores": oracle.num_threads(),
+                                 "seconds_best": min(t_fast), "seconds_mean": sum(t_fast) / 3,
+                                 "what": "bit-identical blocked/OpenMP form of the same loop, full 1024^3, 3 repetitions"}}
         except Exception as ex:
             cpu = {"error": str(ex)[:200]}
 
@@ -200,6 +342,7 @@ def main():
         except Exception as ex:
             vendor = {"error": str(ex)[:200]}
 
+    rep_tf = sorted(to_tflops(x) for x in repeat_ms)
     out = {
         "metric": "FP8 GEMM TFLOPS at 8192^3 e4m3 (skinny M=16 HBM GB/s in `skinny`)",
         "value": tflops,
@@ -217,11 +360,28 @@ def main():
         "config": {"workload": "M=N=K=8192, A row-major MxK e4m3, B stored NxK e4m3, C fp32 row-major",
                    "entry_point": "fp8gemm_launch (automatic kernel choice), stages=2"},
         "frac_of_fp8_peak": tflops / PEAK_FP8_TFLOPS,
+        "settle": {"what": "untimed launches before --warmup, in blocks of %d until three successive blocks agree "
+                           "within %d %% (cap %.0f s): the chip's power management needs continuous load to settle"
+                           % (SETTLE_BLOCK, round((SETTLE_AGREE - 1) * 100), SETTLE_CAP_S),
+                   "settle_launches": SETTLE_BLOCK * len(settle_blocks),
+                   "last_block_tflops": to_tflops(settle_blocks[-1]),
+                   "slowest_block_tflops": to_tflops(max(settle_blocks))},
+        "cold_burst": {"what": "the first %d launches after the chip sat idle" % SETTLE_BLOCK,
+                       "ms_per_step": settle_blocks[0], "tflops": to_tflops(settle_blocks[0]),
+                       "frac_of_fp8_peak": to_tflops(settle_blocks[0]) / PEAK_FP8_TFLOPS},
+        "repeats": {"what": "five more blocks of `steps` launches right after the timed one",
+                    "tflops_median": rep_tf[2], "tflops_min": rep_tf[0], "tflops_max": rep_tf[-1]},
+        "board": sampler.summary(),
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / PEAK_FP8_TFLOPS, "traffic": TRAFFIC_BYTES_8192,
+                     "traffic_source": "constant from the rocprofv3 --pmc summary under profiles/ "
+                                       "(FETCH_SIZE %d KiB x %.1f + WRITE_SIZE %d KiB x %.1f), not read in this run"
+                                       % (TRAFFIC_8192["fetch_kib"], TRAFFIC_8192["fetch_scale"],
+                                          TRAFFIC_8192["write_kib"], TRAFFIC_8192["write_scale"]),
                      "algorithmic_flops": flops, "algorithmic_bytes": alg_bytes,
                      "kernel_ms": ms},
         "skinny": skinny,
+        "llm_shapes": llm,
         "parity": parity,
         "cpu_baseline": cpu,
         "vendor": vendor,

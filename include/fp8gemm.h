@@ -84,13 +84,20 @@ int fp8gemm_launch_ex(int m, int k, int n, const void *a, int a_fmt, const void 
                       void *out, int out_type, float alpha, const float *a_scale, const float *b_scale,
                       void *stream);
 
+/*
+ * ---- Internal: testing and tuning hooks --------------------------------------------
+ * fp8gemm_launch_algo, fp8gemm_launch_tuned, fp8gemm_num_variants, fp8gemm_plan and
+ * fp8gemm_tile_order expose the kernel families, their compiled variants and the planner
+ * to the test suite and the tuning sweeps.  They are not part of the drop-in surface:
+ * variant numbers, plan encodings and the set of variants change between versions.
+ */
 /* As fp8gemm_launch, but forces one kernel family (FP8GEMM_ALGO_*).  Returns
  * hipErrorInvalidValue when the family cannot run the shape. */
 int fp8gemm_launch_algo(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
                         float *out, int stages, int algo, void *stream);
 
 /*
- * Tuning hook with no counterpart in the reference: forces a kernel family
+ * Internal tuning hook with no counterpart in the reference: forces a kernel family
  * and one of its compiled shape variants (0 .. fp8gemm_num_variants(algo)-1,
  * -1 = the default for the shape).  For FP8GEMM_ALGO_SKINNY, variant may add
  * 16 * columns-per-wave/16 to override the planned column count per wave; for
@@ -125,12 +132,38 @@ int fp8gemm_plan(int m, int k, int n, int stages, int plan[4]);
  */
 int fp8gemm_tile_order(int m, int k, int n, int bm, int bn, int index, int *tile_row, int *tile_col);
 
-/* Bytes of device scratch (partial sums of K slices) the library keeps cached
- * per device for a shape (0 when the shape needs none).  The scratch is the
- * only allocation the library ever makes; it is grown on demand, reused by
- * later calls and shared by all streams of the device, so calls that overlap
- * on one device and both need it must be ordered by the caller. */
-size_t fp8gemm_scratch_bytes(int m, int k, int n);   /* for the stage-2 plan; the stage-4 plan cuts K the same way */
+/*
+ * Device scratch.  A shape whose plan cuts K into slices needs device memory for the
+ * slices' partial sums between its two kernels; fp8gemm_scratch_bytes tells how much
+ * (0 when the shape needs none: 8192^3, M=16 N=28672 K=8192, ...; the figure is for the
+ * stage-2 plan, the stage-4 plan cuts K the same way).  It is the only device memory the
+ * library ever allocates.  The reference's launchers are stateless and re-entrant
+ * (GEMM/src/gemm.cu:263-277); to keep that contract the scratch is held per (device,
+ * stream): calls on one stream are ordered by the stream, calls on different streams
+ * never share a buffer and may overlap freely, from one host thread or several.  A
+ * stream's buffer is allocated on its first K-sliced call (hipMalloc), reused by later
+ * calls, and replaced by a larger one when a shape needs more; the smaller buffer is kept
+ * and handed to another stream once the work queued on it has finished.  No call waits
+ * for the device and none frees memory.  fp8gemm_release_scratch synchronises the current
+ * device and frees everything held for it; fp8gemm_scratch_held_bytes reports what is held.
+ * hipMalloc is illegal while a stream is being captured into a graph: capture only shapes
+ * that need no scratch or whose stream already owns a large enough buffer, or call
+ * fp8gemm_launch_ws.
+ */
+size_t fp8gemm_scratch_bytes(int m, int k, int n);
+int fp8gemm_release_scratch(void);
+size_t fp8gemm_scratch_held_bytes(void);
+
+/*
+ * fp8gemm_launch with the scratch supplied by the caller: `workspace` is device memory of
+ * `workspace_bytes` bytes, 16-byte aligned, that the call's kernels may overwrite and that
+ * must stay untouched until they have run (NULL / 0 for shapes that need none).  Returns
+ * hipErrorOutOfMemory (2) without launching anything when the shape needs more than
+ * workspace_bytes (see fp8gemm_scratch_bytes).  The library allocates nothing in this call.
+ * No counterpart in the reference, whose kernels need no workspace.
+ */
+int fp8gemm_launch_ws(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
+                      float *out, int stages, void *workspace, size_t workspace_bytes, void *stream);
 
 /* Text for a return code (hipGetErrorString). */
 const char *fp8gemm_error_string(int code);

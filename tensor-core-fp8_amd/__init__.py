@@ -66,6 +66,12 @@ def lib():
         fn.argtypes = [ci, ci, ci, vp, vp, vp]
     L.fp8gemm_launch.restype = ci
     L.fp8gemm_launch.argtypes = [ci, ci, ci, vp, ci, vp, ci, vp, ci, vp]
+    L.fp8gemm_launch_ws.restype = ci
+    L.fp8gemm_launch_ws.argtypes = [ci, ci, ci, vp, ci, vp, ci, vp, ci, vp, ctypes.c_size_t, vp]
+    L.fp8gemm_release_scratch.restype = ci
+    L.fp8gemm_release_scratch.argtypes = []
+    L.fp8gemm_scratch_held_bytes.restype = ctypes.c_size_t
+    L.fp8gemm_scratch_held_bytes.argtypes = []
     L.fp8gemm_launch_ex.restype = ci
     L.fp8gemm_launch_ex.argtypes = [ci, ci, ci, vp, ci, vp, ci, vp, ci, ctypes.c_float, vp, vp, vp]
     L.fp8gemm_launch_algo.restype = ci

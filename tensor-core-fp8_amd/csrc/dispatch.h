@@ -1,0 +1,317 @@
+// Kernel choice and launch for one operand pairing: everything between the validated
+// arguments of the C ABI and hipLaunchKernelGGL.  Included by dispatch_pair.hip, which is
+// compiled once per pairing so that the four pairings build in parallel.
+#ifndef FP8GEMM_DISPATCH_H
+#define FP8GEMM_DISPATCH_H
+
+#include <atomic>
+
+#include "kernel_direct.h"
+#include "kernel_ptile.h"
+#include "kernel_skinny.h"
+#include "kernel_tile.h"
+#include "plan.h"
+
+namespace fp8gemm_detail {
+
+// ------------------------------------------------------------------ variants
+// Tiled kernel shapes: <BM, BN, BK, waves_m, waves_n, stages, swizzle>.
+using TileP2 = TileShape<256, 256, 128, 2, 2, 2, 3>;  // persistent, 2 x 64 KiB ring, 128x128 per wave
+using TileP2h = TileShape<256, 256, 128, 2, 2, 2, 3, true>;   // the same on v_mfma_f32_16x16x128_f8f6f4
+using TileT2h = TileShape<192, 256, 128, 2, 2, 2, 3, true>;   // 192 x 256 on that MFMA
+using TileP4 = TileShape<256, 256, 64, 2, 2, 4, 2>;   // persistent, 4 x 32 KiB ring
+using TileP8 = TileShape<256, 256, 128, 2, 4, 2, 3>;  // persistent, 8 waves, 128x64 per wave
+using TileS2 = TileShape<128, 128, 128, 2, 2, 2, 3>;  // one tile per workgroup, for small problems
+using TileS4 = TileShape<128, 128, 128, 2, 2, 4, 3>;
+using TileH3 = TileShape<128, 256, 128, 2, 2, 3, 3>;  // persistent, half-height tile, 3 x 48 KiB ring
+using TileQ2 = TileShape<128, 128, 128, 2, 2, 2, 3>;  // persistent, quarter tile
+using TileS64 = TileShape<128, 128, 64, 2, 2, 4, 2>;  // one tile per workgroup, 64-byte K tiles
+using TileW3 = TileShape<256, 128, 128, 2, 2, 3, 3>;  // persistent, half-width tile, 3 x 48 KiB ring
+using TileT2 = TileShape<192, 256, 128, 2, 2, 2, 3>;  // persistent, three-quarter-height tile: other tile counts
+// the 4-deep rings of 64-byte K tiles behind the stage-4 entry points, same tile shapes
+using TileT4 = TileShape<192, 256, 64, 2, 2, 4, 2>;
+using TileH4 = TileShape<128, 256, 64, 2, 2, 4, 2>;
+using TileQ4 = TileShape<128, 128, 64, 2, 2, 4, 2>;
+
+// Skinny kernel shapes: <MT, TN, BK, stages>.
+template <int MT, int TN>
+using SkinnyV0 = SkinnyShape<MT, TN, 128, 5>;
+template <int MT, int TN>
+using SkinnyV1 = SkinnyShape<MT, TN, 256, 4>;
+template <int MT, int TN>
+using SkinnyV2 = SkinnyShape<MT, TN, 128, 8>;
+template <int MT, int TN>
+using SkinnyV3 = SkinnyShape<MT, TN, 256, 6>;
+template <int MT, int TN>
+using SkinnyV4 = SkinnyShape<MT, TN, 512, 4, 80 * 1024>;
+template <int MT, int TN>
+using SkinnyV5 = SkinnyShape<MT, TN, 1024, 3, 80 * 1024>;
+
+// Raises a kernel's dynamic LDS limit above the 64 KiB default.  Done once per kernel
+// and device (the attribute call costs host time on every launch otherwise); KernelTag
+// is a type unique to the kernel instantiation, it only keys the bookkeeping.
+template <class KernelTag, class Kernel>
+hipError_t allow_lds(Kernel kernel, int bytes)
+{
+    if (bytes <= 64 * 1024) return hipSuccess;
+    static std::atomic<unsigned long long> done{0};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const bool tracked = dev >= 0 && dev < 64;
+    if (tracked && ((done.load(std::memory_order_acquire) >> dev) & 1ull)) return hipSuccess;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess && tracked) done.fetch_or(1ull << dev, std::memory_order_release);
+    return e;
+}
+
+template <class S, int AF, int BF>
+struct TileKernelTag {};
+template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM>
+struct PtileKernelTag {};
+template <class S, int AF, int BF>
+struct SkinnyKernelTag {};
+// ------------------------------------------------------------------ direct
+template <int AF, int BF>
+hipError_t launch_direct(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
+                         const OutSpec &spec, hipStream_t stream)
+{
+    const long gy = (m + 31) / 32, gx = (n + 31) / 32;
+    if (gx * gy > 0x7FFFFFFFL) return hipErrorInvalidValue;       // 2^41 elements of C and more
+    const bool vec_ok = (k % 16 == 0) && ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) % 16 == 0);
+    hipLaunchKernelGGL((gemm_direct_kernel<AF, BF>), dim3((unsigned)(gx * gy)), dim3(64), 0, stream,
+                       m, k, n, a, b, out, (int)gx, vec_ok ? 1 : 0, spec);
+    return hipGetLastError();
+}
+
+// ------------------------------------------------------------------ tiled
+template <class S, int AF, int BF>
+hipError_t launch_tile_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
+                             hipStream_t stream)
+{
+    if (k % S::BK != 0) return hipErrorInvalidValue;
+    const int tiles_m = (m + S::BM - 1) / S::BM;
+    const int tiles_n = (n + S::BN - 1) / S::BN;
+    // XCD-local super-blocks of tiles: 32 CUs per XCD -> blocks of up to 32 tiles,
+    // shaped to balance A-panel and B-panel reuse.
+    int GM = 4, GN = 8;
+    if (tiles_m < GM) { GM = tiles_m; }
+    if (tiles_n < GN) { GN = tiles_n; }
+    const int nb = ((tiles_m + GM - 1) / GM) * ((tiles_n + GN - 1) / GN);
+    const long grid = (long)((nb + 7) / 8) * 8 * GM * GN;
+    auto kernel = gemm_tile_kernel<S, AF, BF>;
+    hipError_t e = allow_lds<TileKernelTag<S, AF, BF>>(kernel, S::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(S::THREADS), S::LDS_BYTES, stream,
+                       m, k, n, a, b, out, tiles_m, tiles_n, GM, GN);
+    return hipGetLastError();
+}
+
+// persistent form: one workgroup per CU walks its share of the work list; the K slices'
+// partial sums go through the scratch buffer and a reduction pass
+template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM>
+hipError_t launch_ptile_work(const PtileWork &w, int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
+                             float *ws, int rotate, const OutSpec &spec, hipStream_t stream)
+{
+    auto kernel = gemm_ptile_kernel<S, AF, BF, KOVER, EX, BSTREAM>;
+    hipError_t e = allow_lds<PtileKernelTag<S, AF, BF, KOVER, EX, BSTREAM>>(kernel, S::PTILE_LDS_BYTES);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * w.slots)), dim3(S::THREADS), S::PTILE_LDS_BYTES, stream,
+                       m, k, n, a, b, out, ws, w.tiles_m, w.tiles_n, w.GM, tile_column_block(w.tiles_n, m, n, k), w.bulk, w.tail,
+                       w.nsplit, w.rounds, rotate, spec);
+    return hipGetLastError();
+}
+
+// STREAM_TOO: this shape is also compiled with non-temporal loads of B, used when C has a
+// single row of tiles (every byte of B is then read by exactly one workgroup)
+template <class S, int AF, int BF, bool KOVER, bool EX, bool STREAM_TOO>
+hipError_t launch_ptile_shape_k(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
+                                int nsplit, bool split_all, int rotate, const OutSpec &spec, Workspace &wsp, hipStream_t stream)
+{
+    if (k % 16 != 0 || k > (1 << 23) || nsplit < 1 || nsplit > (k + S::BK - 1) / S::BK) return hipErrorInvalidValue;
+    const PtileWork w = ptile_work(m, n, S::BM, S::BN, nsplit, split_all);
+    if (!w.ok) return hipErrorInvalidValue;
+    float *ws = nullptr;
+    if (w.nsplit > 1) {
+        void *p = nullptr;
+        hipError_t e = wsp.get(ptile_scratch_bytes(w, S::BM, S::BN), &p);
+        if (e != hipSuccess) return e;
+        ws = static_cast<float *>(p);
+    }
+    hipError_t e;
+    if constexpr (STREAM_TOO && !KOVER) {
+        e = w.tiles_m == 1 ? launch_ptile_work<S, AF, BF, KOVER, EX, true>(w, m, k, n, a, b, out, ws, rotate, spec, stream)
+                           : launch_ptile_work<S, AF, BF, KOVER, EX, false>(w, m, k, n, a, b, out, ws, rotate, spec, stream);
+    } else {
+        e = launch_ptile_work<S, AF, BF, KOVER, EX, false>(w, m, k, n, a, b, out, ws, rotate, spec, stream);
+    }
+    if (e != hipSuccess || w.nsplit == 1) return e;
+    return launch_tile_slices_reduce(ws, out, m, n, k, S::BM, S::BN, w, spec, stream);
+}
+
+// OVERHANG_TOO: this shape is also compiled for a K that is not a multiple of its K tile.
+// EX_TOO: ... and for the extended epilogue (scale, 16-bit output).
+template <class S, int AF, int BF, bool OVERHANG_TOO, bool EX_TOO, bool STREAM_TOO = false>
+hipError_t launch_ptile_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
+                              int nsplit, bool split_all, int rotate, const OutSpec &spec, Workspace &wsp, hipStream_t stream)
+{
+    const bool over = k % S::BK != 0;
+    if (plain_output(spec)) {
+        if (!over)
+            return launch_ptile_shape_k<S, AF, BF, false, false, STREAM_TOO>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+        if constexpr (OVERHANG_TOO)
+            return launch_ptile_shape_k<S, AF, BF, true, false, STREAM_TOO>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+        return hipErrorInvalidValue;
+    }
+    if constexpr (EX_TOO) {
+        if (!over)
+            return launch_ptile_shape_k<S, AF, BF, false, true, STREAM_TOO>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+        if constexpr (OVERHANG_TOO)
+            return launch_ptile_shape_k<S, AF, BF, true, true, STREAM_TOO>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+template <int AF, int BF>
+hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
+                       int variant, int nsplit, bool split_all, int rotate, const OutSpec &spec, Workspace &wsp, hipStream_t stream)
+{
+    const bool persistent = !(variant == 3 || variant == 4 || variant == 7);
+    if (!persistent && nsplit != 1) return hipErrorInvalidValue;   // K slices only in the persistent kernels
+    // the one-tile-per-workgroup kernels write bare fp32 sums only
+    if (!persistent && !plain_output(spec)) return hipErrorInvalidValue;
+    switch (variant) {
+    case 0: return launch_ptile_shape<TileP2, AF, BF, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+    case 1: return launch_ptile_shape<TileP4, AF, BF, true, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+    case 2: return launch_ptile_shape<TileP8, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+    case 3: return launch_tile_shape<TileS2, AF, BF>(m, k, n, a, b, static_cast<float *>(out), stream);
+    case 4: return launch_tile_shape<TileS4, AF, BF>(m, k, n, a, b, static_cast<float *>(out), stream);
+    case 5: return launch_ptile_shape<TileH3, AF, BF, true, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+    case 6: return launch_ptile_shape<TileQ2, AF, BF, true, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+    case 7: return launch_tile_shape<TileS64, AF, BF>(m, k, n, a, b, static_cast<float *>(out), stream);
+    case 8: return launch_ptile_shape<TileW3, AF, BF, false, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+    case 9: return launch_ptile_shape<TileT2, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+    case 10: return launch_ptile_shape<TileT4, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+    case 11: return launch_ptile_shape<TileH4, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+    case 12: return launch_ptile_shape<TileQ4, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+    case 13:
+        if (!p2h_ok(k, nsplit)) return hipErrorInvalidValue;
+        return launch_ptile_shape<TileP2h, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+    case 14:
+        if (!p2h_ok(k, nsplit)) return hipErrorInvalidValue;
+        return launch_ptile_shape<TileT2h, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+// ------------------------------------------------------------------ skinny
+template <class S, int AF, int BF>
+hipError_t launch_skinny_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
+                               int nsplit, const OutSpec &spec, Workspace &wsp, hipStream_t stream)
+{
+    if (m > S::MP || n % S::NP != 0 || nsplit < 1 || k % nsplit != 0 || (k / nsplit) % S::BK != 0)
+        return hipErrorInvalidValue;
+    const int ngroups = n / S::NP;
+    const int kchunk = k / nsplit;
+    void *dst = out;
+    if (nsplit > 1) {
+        void *ws = nullptr;
+        hipError_t e = wsp.get((size_t)nsplit * m * n * sizeof(float), &ws);
+        if (e != hipSuccess) return e;
+        dst = ws;
+    }
+    auto kernel = gemm_skinny_kernel<S, AF, BF>;
+    hipError_t e = allow_lds<SkinnyKernelTag<S, AF, BF>>(kernel, S::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(ngroups * nsplit)), dim3(64), S::LDS_BYTES, stream,
+                       m, k, n, a, b, dst, ngroups, kchunk, nsplit, spec);
+    e = hipGetLastError();
+    if (e != hipSuccess || nsplit == 1) return e;
+    return launch_reduce(static_cast<const float *>(dst), out, (size_t)m * n, nsplit, spec, stream);
+}
+
+template <template <int, int> class V, int AF, int BF>
+hipError_t launch_skinny_mt(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
+                            const SkinnyPlan &p, const OutSpec &spec, Workspace &wsp, hipStream_t stream)
+{
+#define SK(MT, TN) \
+    if (p.mt == MT && p.tn == TN) return launch_skinny_shape<V<MT, TN>, AF, BF>(m, k, n, a, b, out, p.nsplit, spec, wsp, stream);
+    SK(1, 1) SK(1, 2) SK(1, 4)
+    SK(2, 1) SK(2, 2) SK(2, 4)
+    SK(3, 1) SK(3, 2) SK(3, 4)
+    SK(4, 1) SK(4, 2) SK(4, 4)
+#undef SK
+    return hipErrorInvalidValue;
+}
+
+template <int AF, int BF>
+hipError_t launch_skinny(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
+                         const SkinnyPlan &p, const OutSpec &spec, Workspace &wsp, hipStream_t stream)
+{
+    switch (p.variant) {
+    case 0: return launch_skinny_mt<SkinnyV0, AF, BF>(m, k, n, a, b, out, p, spec, wsp, stream);
+    case 1: return launch_skinny_mt<SkinnyV1, AF, BF>(m, k, n, a, b, out, p, spec, wsp, stream);
+    case 2: return launch_skinny_mt<SkinnyV2, AF, BF>(m, k, n, a, b, out, p, spec, wsp, stream);
+    case 3: return launch_skinny_mt<SkinnyV3, AF, BF>(m, k, n, a, b, out, p, spec, wsp, stream);
+    case 4: return launch_skinny_mt<SkinnyV4, AF, BF>(m, k, n, a, b, out, p, spec, wsp, stream);
+    case 5: return launch_skinny_mt<SkinnyV5, AF, BF>(m, k, n, a, b, out, p, spec, wsp, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+template <int AF, int BF>
+hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out, int stages,
+                    int algo, int variant, int nsplit, const OutSpec &spec, Workspace &wsp, hipStream_t stream)
+{
+    const bool aligned = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) % 16) == 0;
+    if (algo == FP8GEMM_ALGO_AUTO) {
+        algo = select_algo(m, k, n);
+        if (!aligned) algo = FP8GEMM_ALGO_DIRECT;
+    }
+    switch (algo) {
+    case FP8GEMM_ALGO_DIRECT:
+        return launch_direct<AF, BF>(m, k, n, a, b, out, spec, stream);
+    case FP8GEMM_ALGO_TILE: {
+        if (!aligned || k % 16 != 0 || k > (1 << 23)) return hipErrorInvalidValue;
+        TilePlan p = plan_tile(m, k, n, stages);
+        if (variant >= 0) {
+            // tuning hook: variant = shape index + 16 * (1 + K-walk rotation mode); a bare
+            // shape index keeps the plan's rotation and runs unsplit unless split_k says otherwise
+            if (variant >= 16) {
+                p.rotate = variant / 16 - 1;
+                if (p.rotate > 2) return hipErrorInvalidValue;
+            }
+            p.variant = variant % 16;
+            p.nsplit = 1;
+            p.split_all = false;
+        }
+        if (nsplit > 0) {          // forced: K slices for every tile
+            p.nsplit = nsplit;
+            p.split_all = true;
+        } else if (nsplit < 0) {   // forced: K slices for the tiles that do not fill a round
+            p.nsplit = -nsplit;
+            p.split_all = false;
+        }
+        return launch_tile<AF, BF>(m, k, n, a, b, out, p.variant, p.nsplit, p.split_all, p.rotate, spec, wsp, stream);
+    }
+    case FP8GEMM_ALGO_SKINNY: {
+        if (!aligned || !skinny_ok(m, k, n)) return hipErrorInvalidValue;
+        SkinnyPlan p = plan_skinny(m, k, n);
+        if (variant >= 0) {
+            // tuning hook: variant = shape_index + 16 * columns-per-wave/16 (0 keeps the plan's)
+            p.variant = variant % 16;
+            if (variant / 16 > 0) p.tn = variant / 16;
+        }
+        if (nsplit > 0) p.nsplit = nsplit;
+        if (nsplit < 0) return hipErrorInvalidValue;
+        return launch_skinny<AF, BF>(m, k, n, a, b, out, p, spec, wsp, stream);
+    }
+    default:
+        return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace fp8gemm_detail
+
+#endif  // FP8GEMM_DISPATCH_H

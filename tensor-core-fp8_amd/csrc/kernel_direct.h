@@ -36,13 +36,14 @@ template <int AF, int BF>
 __global__ __launch_bounds__(64) void gemm_direct_kernel(int M, int K, int N,
                                                          const uint8_t *__restrict__ A,
                                                          const uint8_t *__restrict__ B,
-                                                         void *__restrict__ C, int vec_ok, OutSpec spec)
+                                                         void *__restrict__ C, int tiles_n, int vec_ok, OutSpec spec)
 {
     const int lane = threadIdx.x;
     const int i = lane & 31;
     const int g = lane >> 5;
-    const int m0 = blockIdx.y * 32;
-    const int n0 = blockIdx.x * 32;
+    // a one-dimensional grid (row-major over the tiles of C): neither dimension is capped at 65535 tiles
+    const int m0 = (int)(blockIdx.x / (unsigned)tiles_n) * 32;
+    const int n0 = (int)(blockIdx.x % (unsigned)tiles_n) * 32;
     v16f acc;
     for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
 

@@ -1,0 +1,88 @@
+// Host-side vocabulary shared by the C ABI (fp8gemm.hip) and the per-pairing launch code
+// (dispatch.h): work lists, plans, the workspace of a call.
+#ifndef FP8GEMM_PLAN_H
+#define FP8GEMM_PLAN_H
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <mutex>
+
+#include "device_common.h"
+#include "fp8gemm.h"
+
+namespace fp8gemm_detail {
+
+// tiled kernel shapes: 0 P2, 1 P4, 2 P8, 3 S2, 4 S4, 5 H3, 6 Q2, 7 S64, 8 W3, 9 T2, 10 T4, 11 H4, 12 Q4, 13 P2h, 14 T2h
+constexpr int kNumTileVariants = 15;
+constexpr int kNumSkinnyVariants = 6;
+
+// Work list of the persistent kernel for a tile shape: `bulk` tiles (a multiple of 256)
+// run as whole items, 256 per round; the remaining `tail` tiles are cut into nsplit K
+// slices each.  split_all cuts every tile (bulk = 0); otherwise only the tiles that do
+// not fill a round are cut.
+struct PtileWork {
+    int tiles_m, tiles_n, GM, bulk, tail, nsplit, rounds, slots;
+    bool ok;
+};
+PtileWork ptile_work(int m, int n, int bm, int bn, int nsplit, bool split_all);
+int tile_column_block(int tiles_n, int m, int n, int k);
+size_t ptile_scratch_bytes(const PtileWork &w, int bm, int bn);
+
+// the plain entry points: bare fp32 sums, no scaling
+bool plain_output(const OutSpec &spec);
+// The 16x16x128 forms of the 256 x 256 and 192 x 256 tiles need whole 128-byte K tiles, at least two per
+// work item (a tile, or one of its nsplit K slices).
+bool p2h_ok(int k, int nsplit);
+
+struct SkinnyPlan {
+    int mt, tn, variant, nsplit;
+};
+bool skinny_ok(int m, int k, int n);
+SkinnyPlan plan_skinny(int m, int k, int n);
+int select_algo(int m, int k, int n);
+
+// Which tiled kernel, how many K slices, which K-walk rotation.
+struct TilePlan {
+    int variant, nsplit, rotate;
+    bool split_all;      // K slices for every tile (else only for the tiles that do not fill a round)
+};
+TilePlan plan_tile(int m, int k, int n, int stages);
+size_t tile_plan_scratch_bytes(int m, int n, const TilePlan &p);
+
+// Where the partial sums of one call's K slices go: a buffer of the per-(device, stream)
+// pool, or a fixed buffer (the caller's workspace, or the static array).  A pooled
+// workspace keeps the pool locked from its first lookup until it goes out of scope, i.e.
+// until the call's kernels are enqueued.
+class Workspace {
+public:
+    static Workspace pooled(hipStream_t stream) { return Workspace(stream, nullptr, 0, true); }
+    static Workspace fixed(void *ptr, size_t bytes) { return Workspace(nullptr, ptr, bytes, false); }
+    hipError_t get(size_t need, void **out);
+
+private:
+    Workspace(hipStream_t stream, void *ptr, size_t bytes, bool pooled)
+        : stream_(stream), ptr_(ptr), bytes_(bytes), pooled_(pooled) {}
+    hipStream_t stream_;
+    void *ptr_;
+    size_t bytes_;
+    bool pooled_;
+    std::unique_lock<std::mutex> lock_;
+};
+
+// out[i] = sum over the nsplit planes of ws, on `stream`
+hipError_t launch_reduce(const float *ws, void *out, size_t count, int nsplit, const OutSpec &spec, hipStream_t stream);
+// sum of the K slices of the persistent kernel's tail tiles (scratch slots of bm x bn floats) into C
+hipError_t launch_tile_slices_reduce(const float *ws, void *out, int m, int n, int k, int bm, int bn, const PtileWork &w,
+                                     const OutSpec &spec, hipStream_t stream);
+
+// Validated operands -> kernel choice and launch for one operand pairing (AF, BF: 0 = E4M3,
+// 1 = E5M2).  Each pairing is compiled in a translation unit of its own (dispatch_pair.hip).
+template <int AF, int BF>
+hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out, int stages,
+                    int algo, int variant, int nsplit, const OutSpec &spec, Workspace &wsp, hipStream_t stream);
+
+}  // namespace fp8gemm_detail
+
+#endif  // FP8GEMM_PLAN_H

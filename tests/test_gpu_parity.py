@@ -27,28 +27,31 @@ def run_gpu(pkg, A, fa, B, fb, **kw):
     return out.cpu().numpy()
 
 
-def mfma_window_term(oracle, A, fa, B, fb, block=64):
+def mfma_window_term(oracle, A, fa, B, fb, block=8):
     """Extra error the f8f6f4 MFMA can add on top of reordered fp32 summation.
 
-    Measured on MI355X: inside one MFMA the products of a K block are aligned to
-    the largest product exponent of the block and only ~14 bits below it are
-    kept (2^16 + 2^3 survives, 2^16 + 2^2 does not); between MFMAs the sum is
-    plain fp32.  So each block can lose up to one unit of 2^-13 * max|product|
-    per product.
+    Measured on MI355X and pinned by tests/test_gpu_mfma_numerics.py: the products of 8
+    consecutive K bytes are added as a group, aligned to the group's largest product, keeping
+    13 binary places below its leading bit (2^16 + 2^3 survives, 2^16 + 2^2 does not); groups,
+    MFMAs and K tiles are added in plain fp32.  So each group can lose up to 2^-13 of its
+    largest product per product.  Returned: 2^-13 * sum over groups of (8 * an upper bound of
+    the group's largest |a*b|).
     """
-    a = oracle.decode(A, fa).astype(np.float64)
-    b = oracle.decode(B, fb).astype(np.float64)
+    a = np.abs(oracle.decode(A, fa).astype(np.float64))
+    b = np.abs(oracle.decode(B, fb).astype(np.float64))
     M, K = a.shape
-    N = b.shape[0]
-    term = np.zeros((M, N))
-    for k0 in range(0, K, block):
-        pa = np.abs(a[:, None, k0:k0 + block])
-        pb = np.abs(b[None, :, k0:k0 + block])
-        term += (pa * pb).max(axis=2) * min(block, K - k0)
-    return term * 2.0 ** -13
+    pad = (-K) % block
+    if pad:
+        a = np.pad(a, ((0, 0), (0, pad)))
+        b = np.pad(b, ((0, 0), (0, pad)))
+    # largest |a*b| of a group <= (largest |a| of the group) * (largest |b| of the group):
+    # a matrix product of the group maxima instead of a pass over every product
+    amax = a.reshape(M, -1, block).max(axis=2)
+    bmax = b.reshape(b.shape[0], -1, block).max(axis=2)
+    return (amax @ bmax.T) * block * 2.0 ** -13
 
 
-def assert_within_bound(oracle, C, A, fa, B, fb, rows=None, hw_term=False, block=64):
+def assert_within_bound(oracle, C, A, fa, B, fb, rows=None, hw_term=False, block=8):
     K = A.shape[1]
     Cref, S = oracle.gemm(A, fa, B, fb, rows=rows, with_scale=True)
     got = C if rows is None else C[rows]
@@ -56,7 +59,8 @@ def assert_within_bound(oracle, C, A, fa, B, fb, rows=None, hw_term=False, block
     err = np.abs(got.astype(np.float64) - Cref.astype(np.float64))
     tol = oracle.tolerance(K, S)
     if hw_term:
-        tol = tol + mfma_window_term(oracle, A, fa, B, fb, block=block)
+        term = mfma_window_term(oracle, A, fa, B, fb, block=block)
+        tol = tol + (term if rows is None else term[rows])
     worst = float((err / np.maximum(tol, 1e-300)).max())
     assert (err <= tol).all(), "worst err/tol = %g" % worst
     return worst
@@ -107,18 +111,22 @@ def test_normal_inputs_within_fp32_reordering_bound(pkg, oracle, fa, fb, algo, s
     assert worst < 0.25
 
 
+@pytest.mark.parametrize("fa,fb", PAIRS)
 @pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12])
 @pytest.mark.parametrize("shape", [(256, 256, 256), (300, 512, 200), (1000, 1024, 900), (513, 384, 257), (64, 128, 2048)])
-def test_every_tile_variant(pkg, oracle, variant, shape):
+def test_every_tile_variant(pkg, oracle, variant, shape, fa, fb):
     """Each compiled shape of the tiled kernels (persistent and one-tile-per-workgroup),
-    on shapes that overhang the tile in m and n, for a mixed pairing."""
+    on shapes that overhang the tile in m and n, for all four pairings."""
     M, K, N = shape
-    rng = np.random.default_rng(zlib.crc32(repr((variant, shape)).encode()))
-    A = random_codes(rng, (M, K), 0)
-    B = random_codes(rng, (N, K), 1)
-    B = np.where(((B >> 2) & 0x1F) > 24, B & 0x83 | 0x3C, B).astype(np.uint8)
-    C = run_gpu(pkg, A, 0, B, 1, algo=ALGOS["tile"], variant=variant)
-    assert_within_bound(oracle, C, A, 0, B, 1, hw_term=True)
+    rng = np.random.default_rng(zlib.crc32(repr((variant, shape, fa, fb)).encode()))
+    A = random_codes(rng, (M, K), fa)
+    B = random_codes(rng, (N, K), fb)
+    if fa == 1:
+        A = np.where(((A >> 2) & 0x1F) > 24, A & 0x83 | 0x3C, A).astype(np.uint8)
+    if fb == 1:
+        B = np.where(((B >> 2) & 0x1F) > 24, B & 0x83 | 0x3C, B).astype(np.uint8)
+    C = run_gpu(pkg, A, fa, B, fb, algo=ALGOS["tile"], variant=variant)
+    assert_within_bound(oracle, C, A, fa, B, fb, hw_term=True)
 
 
 @pytest.mark.parametrize("shape", [(256, 256, 256), (300, 512, 200), (1000, 1024, 900), (513, 768, 257), (64, 256, 2048),
@@ -138,7 +146,7 @@ def test_tile_variant_on_16x16x128_mfma(pkg, oracle, variant, fa, fb, shape):
     if fb == 1:
         B = np.where(((B >> 2) & 0x1F) > 24, B & 0x83 | 0x3C, B).astype(np.uint8)
     C = run_gpu(pkg, A, fa, B, fb, algo=ALGOS["tile"], variant=variant)
-    assert_within_bound(oracle, C, A, fa, B, fb, hw_term=True, block=128)     # one MFMA spans 128 of K here
+    assert_within_bound(oracle, C, A, fa, B, fb, hw_term=True)
 
 
 @pytest.mark.parametrize("variant", [13, 14])
@@ -266,14 +274,57 @@ def test_decode_through_mfma_is_bit_exact(pkg, oracle, fa, fb, algo):
     expect = oracle.decode(B, fb)[:, ks].T       # (M, N)
     assert np.array_equal(C.view(np.uint32) & 0x7FFFFFFF, expect.view(np.uint32) & 0x7FFFFFFF)
     assert np.array_equal(C, expect)
-    # swapped roles: one-hot B selects entries of A
-    if algo != "skinny":
-        A2 = finite_codes(fa)[rng.integers(0, finite_codes(fa).size, (M, K))]
-        B2 = np.zeros((N, K), dtype=np.uint8)
-        kn = rng.integers(0, K, N)
-        B2[np.arange(N), kn] = one[fb]
-        C2 = run_gpu(pkg, A2, fa, B2, fb, algo=ALGOS[algo])
-        assert np.array_equal(C2, oracle.decode(A2, fa)[:, kn])
+    # swapped roles: one-hot B selects entries of A (every finite code of A's format appears)
+    codes_a = finite_codes(fa)
+    A2 = codes_a[rng.integers(0, codes_a.size, (M, K))]
+    A2[:, 0] = np.resize(codes_a, M)
+    A2[0, :codes_a.size] = codes_a[:K]
+    B2 = np.zeros((N, K), dtype=np.uint8)
+    kn = rng.integers(0, K, N)
+    kn[:K] = rng.permutation(K)[:min(K, N)]
+    B2[np.arange(N), kn] = one[fb]
+    C2 = run_gpu(pkg, A2, fa, B2, fb, algo=ALGOS[algo])
+    assert np.array_equal(C2, oracle.decode(A2, fa)[:, kn])
+
+
+@pytest.mark.parametrize("algo,variant", [("tile", 13), ("tile", 14), ("tile", 5), ("tile", 6), ("tile", 8), ("tile", 1)])
+@pytest.mark.parametrize("fa,fb", PAIRS)
+def test_decode_through_mfma_every_persistent_form(pkg, oracle, fa, fb, algo, variant):
+    """The same bit-exact selection test for the persistent tile shapes the planner uses
+    (both MFMA shapes, 2-, 3- and 4-deep rings): one-hot A selects codes of B and one-hot B
+    selects codes of A, K = 512 so that the 16x16x128 forms see four K tiles."""
+    one = {0: 0x38, 1: 0x3C}
+    M, K, N = 384, 512, 512
+    rng = np.random.default_rng(1000 + variant)
+    codes_a, codes_b = finite_codes(fa), finite_codes(fb)
+    ks = rng.integers(0, K, M)
+    A = np.zeros((M, K), dtype=np.uint8)
+    A[np.arange(M), ks] = one[fa]
+    B = codes_b[rng.integers(0, codes_b.size, (N, K))]
+    B[:, ks[0]] = np.resize(codes_b, N)
+    C = run_gpu(pkg, A, fa, B, fb, algo=ALGOS[algo], variant=variant)
+    assert np.array_equal(C, oracle.decode(B, fb)[:, ks].T)
+    A2 = codes_a[rng.integers(0, codes_a.size, (M, K))]
+    A2[:, 3] = np.resize(codes_a, M)
+    kn = rng.integers(0, K, N)
+    kn[0] = 3
+    B2 = np.zeros((N, K), dtype=np.uint8)
+    B2[np.arange(N), kn] = one[fb]
+    C2 = run_gpu(pkg, A2, fa, B2, fb, algo=ALGOS[algo], variant=variant)
+    assert np.array_equal(C2, oracle.decode(A2, fa)[:, kn])
+
+
+def test_tall_general_kernel_shape_beyond_65535_row_tiles(pkg, oracle):
+    """m = 3,000,000 rows with a K that only the general kernel takes (k % 16 != 0): the grid
+    is one-dimensional, so neither tile count is capped at 65535."""
+    M, K, N = 3_000_000, 8, 16
+    assert pkg.lib().fp8gemm_select_algo(M, K, N) == ALGOS["direct"]
+    rng = np.random.default_rng(77)
+    vals = np.arange(-8, 9, dtype=np.float32)           # small integers: every sum is exact
+    Af = vals[rng.integers(0, vals.size, (M, K))]
+    Bf = vals[rng.integers(0, vals.size, (N, K))]
+    C = run_gpu(pkg, oracle.encode(Af, 0), 0, oracle.encode(Bf, 1), 1)
+    assert np.array_equal(C, Af @ Bf.T)
 
 
 @pytest.mark.parametrize("algo,shape", [("direct", (96, 200, 64)), ("tile", (256, 1024, 256)), ("skinny", (48, 1024, 128))])
@@ -327,8 +378,8 @@ def test_column_blocked_tile_numbering(pkg, oracle, variant, split):
 
 def test_scratch_grows_and_is_reused_across_calls_and_streams(pkg, oracle):
     """Calls that need the partial-sum scratch, in growing and shrinking order, on the default
-    stream and on a side stream (ordered by the caller): every result is right, before and
-    after the scratch has been reallocated."""
+    stream and on a side stream: every result is right, before and after a stream's buffer
+    has been replaced by a larger one."""
     import torch
     shapes = [(256, 8192, 1024), (256, 8192, 2048), (256, 8192, 1024), (300, 6144, 1000), (256, 8192, 2048)]
     side = torch.cuda.Stream()
@@ -350,6 +401,78 @@ def test_scratch_grows_and_is_reused_across_calls_and_streams(pkg, oracle):
             torch.cuda.synchronize()
         worst = assert_within_bound(oracle, out.cpu().numpy(), A, 0, B, 0)
         assert worst < 0.25, (idx, worst)
+    assert pkg.lib().fp8gemm_scratch_held_bytes() >= max(need)
+    assert pkg.lib().fp8gemm_release_scratch() == 0
+    assert pkg.lib().fp8gemm_scratch_held_bytes() == 0
+
+
+def test_k_sliced_launches_overlap_on_two_streams_without_caller_ordering(pkg, oracle):
+    """Two streams, each queueing K-sliced GEMMs (which go through the scratch and the
+    reduction kernel) back to back with no ordering between the streams and no host
+    synchronisation: the launch functions are re-entrant like the reference's
+    (GEMM/src/gemm.cu:263-277), so every output is right.  The grids are small enough
+    (64 workgroups on 256 CUs) for kernels of the two streams to run side by side; one
+    stream also grows its buffer in the middle of the sequence."""
+    import torch
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    shapes = [[(256, 8192, 1024), (128, 8192, 2048), (256, 8192, 1024), (256, 8192, 2048)],
+              [(128, 8192, 4096), (256, 8192, 1024), (300, 6144, 1000), (256, 8192, 1024)]]
+    for sh in shapes[0] + shapes[1]:
+        assert pkg.plan(*sh)[2] > 1                    # every shape here is cut into K slices
+    cases = [[], []]
+    for s in range(2):
+        for idx in range(12):
+            M, K, N = shapes[s][idx % 4]
+            A = pkg.fill((M, K), 0, seed=0xA11CE + 300 + 50 * s + idx, dist="normal", sigma=2.0)
+            B = pkg.fill((N, K), 1, seed=0xB0B + 300 + 50 * s + idx, dist="normal", sigma=2.0)
+            cases[s].append((A, B, torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(),
+                             torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")))
+    torch.cuda.synchronize()
+    for idx in range(12):
+        for s in range(2):
+            A, B, dA, dB, out = cases[s][idx]
+            pkg.gemm(dA, dB, out=out, a_fmt=0, b_fmt=1, stream=streams[s])
+    torch.cuda.synchronize()
+    for s in range(2):
+        for A, B, dA, dB, out in cases[s]:
+            worst = assert_within_bound(oracle, out.cpu().numpy(), A, 0, B, 1)
+            assert worst < 0.25
+
+
+def test_caller_provided_workspace(pkg, oracle):
+    """fp8gemm_launch_ws: the K slices' partial sums go to the caller's buffer; too small a
+    buffer is refused with hipErrorOutOfMemory before anything is launched; results equal
+    those of fp8gemm_launch bit for bit (same plan, same kernels)."""
+    import torch
+    L = pkg.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    for (M, K, N) in [(256, 8192, 2048), (64, 8192, 2048), (512, 1024, 768)]:
+        need = L.fp8gemm_scratch_bytes(M, K, N)
+        A = pkg.fill((M, K), 0, seed=0xA11CE + 500 + M, dist="normal", sigma=2.0)
+        B = pkg.fill((N, K), 0, seed=0xB0B + 500 + M, dist="normal", sigma=2.0)
+        dA, dB = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+        ref = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        pkg.gemm(dA, dB, out=ref, a_fmt=0, b_fmt=0)
+        got = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        held = L.fp8gemm_scratch_held_bytes()
+        code = L.fp8gemm_launch_ws(M, K, N, dA.data_ptr(), 0, dB.data_ptr(), 0, got.data_ptr(), 2,
+                                   ws.data_ptr() if need else None, need, stream)
+        assert code == 0
+        torch.cuda.synchronize()
+        assert L.fp8gemm_scratch_held_bytes() == held       # the library allocated nothing
+        assert torch.equal(got, ref)
+        assert_within_bound(oracle, got.cpu().numpy(), A, 0, B, 0)
+        if need:
+            got.fill_(float("nan"))
+            assert L.fp8gemm_launch_ws(M, K, N, dA.data_ptr(), 0, dB.data_ptr(), 0, got.data_ptr(), 2,
+                                       ws.data_ptr(), need - 1, stream) == 2
+            assert L.fp8gemm_launch_ws(M, K, N, dA.data_ptr(), 0, dB.data_ptr(), 0, got.data_ptr(), 2,
+                                       None, 0, stream) == 2
+            assert L.fp8gemm_launch_ws(M, K, N, dA.data_ptr(), 0, dB.data_ptr(), 0, got.data_ptr(), 2,
+                                       ws.data_ptr() + 4, need, stream) == 1      # misaligned workspace
+            torch.cuda.synchronize()
+            assert bool(torch.isnan(got).all())             # nothing was launched
 
 
 def test_back_to_back_launches_without_synchronisation(pkg, oracle):
