@@ -85,6 +85,23 @@ int fp8gemm_launch_ex(int m, int k, int n, const void *a, int a_fmt, const void 
                       void *stream);
 
 /*
+ * fp8gemm_launch for callers that cannot allocate: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference
+ * (whose kernels need no scratch).  The partial sums of K slices go to a static device
+ * array of FP8GEMM_NOALLOC_SCRATCH_BYTES bytes that is part of the library's code object
+ * (every GPU the library runs on holds its own copy until the process ends); the call
+ * allocates and frees nothing.  A shape whose plan needs more scratch than the array holds
+ * (see fp8gemm_scratch_bytes) is refused with hipErrorOutOfMemory (2) before anything is
+ * launched.  All calls on one GPU share that GPU's array: calls on one stream are ordered by
+ * the stream, calls that overlap on different streams of one GPU race on it and must be
+ * ordered by the caller.  Nothing in the array has to start at zero (every slot a call reads
+ * has been written by that call), so none of it is ever cleared.
+ */
+#define FP8GEMM_NOALLOC_SCRATCH_BYTES ((size_t)64 << 20)
+int fp8gemm_launch_noalloc(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
+                           float *out, int stages, void *stream);
+
+/*
  * ---- Internal: testing and tuning hooks --------------------------------------------
  * fp8gemm_launch_algo, fp8gemm_launch_tuned, fp8gemm_num_variants, fp8gemm_plan and
  * fp8gemm_tile_order expose the kernel families, their compiled variants and the planner

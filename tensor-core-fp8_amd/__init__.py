@@ -68,6 +68,8 @@ def lib():
     L.fp8gemm_launch.argtypes = [ci, ci, ci, vp, ci, vp, ci, vp, ci, vp]
     L.fp8gemm_launch_ws.restype = ci
     L.fp8gemm_launch_ws.argtypes = [ci, ci, ci, vp, ci, vp, ci, vp, ci, vp, ctypes.c_size_t, vp]
+    L.fp8gemm_launch_noalloc.restype = ci
+    L.fp8gemm_launch_noalloc.argtypes = [ci, ci, ci, vp, ci, vp, ci, vp, ci, vp]
     L.fp8gemm_release_scratch.restype = ci
     L.fp8gemm_release_scratch.argtypes = []
     L.fp8gemm_scratch_held_bytes.restype = ctypes.c_size_t

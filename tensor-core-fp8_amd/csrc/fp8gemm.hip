@@ -50,6 +50,33 @@ struct HipScratchBackend {
 };
 ScratchPool<HipScratchBackend> g_pool;
 
+// The scratch array of the entry point that allocates nothing: part of the code object,
+// so every device the library runs on holds its own copy from the moment the code is loaded.
+constexpr size_t kStaticScratchBytes = FP8GEMM_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+void *g_static_scratch[kMaxDevices];       // device address of `scratch`, per device
+std::mutex g_static_scratch_mutex;
+
+// Device address of this device's copy of `scratch` (the array's name is only a host-side
+// handle; kernels and runtime calls take the address looked up here).
+hipError_t static_scratch_address(void **out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+    if (!g_static_scratch[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        g_static_scratch[dev] = p;
+    }
+    *out = g_static_scratch[dev];
+    return hipSuccess;
+}
+
 }  // namespace
 
 hipError_t Workspace::get(size_t need, void **out)
@@ -344,6 +371,16 @@ int fp8gemm_launch_ws(int m, int k, int n, const void *a, int a_fmt, const void 
 {
     if (workspace && reinterpret_cast<uintptr_t>(workspace) % 16 != 0) return (int)hipErrorInvalidValue;
     Workspace wsp = Workspace::fixed(workspace, workspace ? workspace_bytes : 0);
+    return launch_checked(m, k, n, a, a_fmt, b, b_fmt, out, stages, FP8GEMM_ALGO_AUTO, -1, 0, stream, kPlainOut, wsp);
+}
+
+int fp8gemm_launch_noalloc(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
+                           float *out, int stages, void *stream)
+{
+    void *ptr = nullptr;
+    const hipError_t e = static_scratch_address(&ptr);
+    if (e != hipSuccess) return (int)e;
+    Workspace wsp = Workspace::fixed(ptr, kStaticScratchBytes);
     return launch_checked(m, k, n, a, a_fmt, b, b_fmt, out, stages, FP8GEMM_ALGO_AUTO, -1, 0, stream, kPlainOut, wsp);
 }
 
