@@ -68,18 +68,30 @@ int fp8gemm_launch(int m, int k, int n, const void *a, int a_fmt, const void *b,
 
 /*
  * Extended epilogue, with no counterpart in the reference's gemm:: API; it covers what the
- * reference's vendor-library sample passes to cuBLASLt next to the operands (host alpha,
- * device pointers to per-tensor scales of A and B: GEMM/src/cublas.cu:9-16, 41-42) and a
- * 16-bit output:
- *     out[i*n+j] = cast_out_type( alpha * a_scale * b_scale * sum_t a[i*k+t] * b[j*k+t] )
- * with the sum accumulated in fp32 as in fp8gemm_launch, the scaling done in fp32 and one
- * rounding to nearest even at the end.  out_type: FP8GEMM_OUT_F32 (float), FP8GEMM_OUT_BF16,
- * FP8GEMM_OUT_F16 (2-byte elements).  a_scale / b_scale: device pointers to one float each,
- * read by the kernel when it runs, or NULL for 1.  Pure overwrite: out is never read (no beta).
+ * reference's vendor-library sample hands to cuBLASLt next to the operands
+ * (GEMM/src/cublas.cu:9-23, 41-46; GEMM/include/helper.h:84, 125, 159-160: host alpha and
+ * beta, device pointers to per-tensor scales of A, B, C and D, a device pointer that receives
+ * the largest magnitude of the output) and 16-bit matrices:
+ *
+ *     y[i*n+j] = alpha * a_scale * b_scale * sum_t a[i*k+t] * b[j*k+t]  +  beta * c_scale * c[i*n+j]
+ *     *amax_d  = max_ij |y[i*n+j]|                      (before d_scale; NaNs do not enter)
+ *     d[i*n+j] = cast_d_type( d_scale * y[i*n+j] )      (one rounding to nearest even)
+ *
+ * The sum is accumulated in fp32 as in fp8gemm_launch and all epilogue arithmetic is fp32.
+ * d_type / c_type: FP8GEMM_OUT_F32 (float), FP8GEMM_OUT_BF16, FP8GEMM_OUT_F16 (2-byte
+ * elements).  a_scale, b_scale, c_scale, d_scale: device pointers to one float each, read by
+ * the kernel when it runs, or NULL for 1.  c: device matrix m x n row-major of c_type, or NULL
+ * (then beta and c_scale are ignored and nothing is read); c may be d itself when both have
+ * the same type (in place).  amax_d: device pointer to one float that the call overwrites, or
+ * NULL.  fp8gemm_launch_ex is the subset without c, d_scale and amax_d.
  */
 #define FP8GEMM_OUT_F32 0
 #define FP8GEMM_OUT_BF16 1
 #define FP8GEMM_OUT_F16 2
+int fp8gemm_launch_epilogue(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
+                            void *d, int d_type, float alpha, float beta, const void *c, int c_type,
+                            const float *a_scale, const float *b_scale, const float *c_scale, const float *d_scale,
+                            float *amax_d, void *stream);
 int fp8gemm_launch_ex(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
                       void *out, int out_type, float alpha, const float *a_scale, const float *b_scale,
                       void *stream);

@@ -74,6 +74,9 @@ def lib():
     L.fp8gemm_release_scratch.argtypes = []
     L.fp8gemm_scratch_held_bytes.restype = ctypes.c_size_t
     L.fp8gemm_scratch_held_bytes.argtypes = []
+    L.fp8gemm_launch_epilogue.restype = ci
+    L.fp8gemm_launch_epilogue.argtypes = [ci, ci, ci, vp, ci, vp, ci, vp, ci, ctypes.c_float, ctypes.c_float, vp, ci,
+                                          vp, vp, vp, vp, vp, vp]
     L.fp8gemm_launch_ex.restype = ci
     L.fp8gemm_launch_ex.argtypes = [ci, ci, ci, vp, ci, vp, ci, vp, ci, ctypes.c_float, vp, vp, vp]
     L.fp8gemm_launch_algo.restype = ci
@@ -235,6 +238,35 @@ def gemm_ex(a, b, out_dtype=None, out=None, alpha=1.0, a_scale=None, b_scale=Non
                                   out.data_ptr(), code, float(alpha),
                                   None if a_scale is None else a_scale.data_ptr(),
                                   None if b_scale is None else b_scale.data_ptr(), _stream_handle(stream)))
+    return out
+
+
+def gemm_epilogue(a, b, out_dtype=None, out=None, alpha=1.0, beta=0.0, c=None, a_scale=None, b_scale=None,
+                  c_scale=None, d_scale=None, amax=None, a_fmt=None, b_fmt=None, stream=None):
+    """d = cast(d_scale * (alpha * a_scale * b_scale * sum_k a b + beta * c_scale * c)) through
+    fp8gemm_launch_epilogue; amax (a one-element float32 device tensor) receives the largest
+    magnitude before d_scale.  c: (m, n) device tensor of float32 / bfloat16 / float16 or None;
+    the scales are one-element float32 device tensors or None."""
+    import torch
+    if not (a.is_cuda and b.is_cuda and a.is_contiguous() and b.is_contiguous()):
+        raise Fp8GemmError("operands must be contiguous device tensors")
+    m, k = a.shape
+    n, k2 = b.shape
+    if k != k2:
+        raise Fp8GemmError("inner dimensions differ: %d vs %d" % (k, k2))
+    codes = {torch.float32: OUT_F32, torch.bfloat16: OUT_BF16, torch.float16: OUT_F16}
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype or torch.float32, device=a.device)
+    for s in (a_scale, b_scale, c_scale, d_scale, amax):
+        if s is not None and not (s.is_cuda and s.dtype == torch.float32 and s.numel() == 1):
+            raise Fp8GemmError("scales and amax are one-element float32 device tensors")
+    if c is not None and not (c.is_cuda and c.is_contiguous() and tuple(c.shape) == (m, n)):
+        raise Fp8GemmError("c must be a contiguous (m, n) device tensor")
+    ptr = lambda t: None if t is None else t.data_ptr()
+    check(lib().fp8gemm_launch_epilogue(m, k, n, a.data_ptr(), _fmt_of(a, a_fmt), b.data_ptr(), _fmt_of(b, b_fmt),
+                                        out.data_ptr(), codes[out.dtype], float(alpha), float(beta), ptr(c),
+                                        codes[c.dtype] if c is not None else OUT_F32, ptr(a_scale), ptr(b_scale),
+                                        ptr(c_scale), ptr(d_scale), ptr(amax), _stream_handle(stream)))
     return out
 
 

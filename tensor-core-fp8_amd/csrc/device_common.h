@@ -66,10 +66,17 @@ __host__ __device__ __forceinline__ void tile_of_number(int g, int tiles_m, int 
     tm = strip * GM + rem - col * h;
 }
 
-// What a kernel does with a finished fp32 sum: multiply by alpha * a_scale * b_scale and
-// store as fp32, bf16 or fp16 (round to nearest even).  The scale pointers are device
-// pointers to one float each, or null for 1.  The plain entry points use {1, null, null,
-// fp32}: the multiplication by 1.0f is exact, results are the bare sums.
+// What a kernel does with a finished fp32 sum s of element i:
+//     y = alpha * a_scale * b_scale * s  +  beta * c_scale * C[i]        (C read only when given)
+//     amax = max(amax, |y|)                                              (only when given)
+//     D[i] = cast_type(d_scale * y)                                      (round to nearest even)
+// -- what the reference's vendor-library sample hands to cuBLASLt next to the operands
+// (GEMM/src/cublas.cu:9-23, 41-46: host alpha and beta, device pointers to per-tensor scales
+// of A, B, C and D, a device pointer for the largest magnitude of the output).  The scale
+// pointers point to one float each, or are null for 1; c is a device matrix laid out like D
+// (m x n row-major) of type c_type, or null (then beta is not used and C is never read); c may
+// be D itself.  The plain entry points use {1, null, null, fp32, ...nothing else}: the
+// multiplication by 1.0f is exact, results are the bare sums.
 #define FP8GEMM_DEV_OUT_F32 0
 #define FP8GEMM_DEV_OUT_BF16 1
 #define FP8GEMM_DEV_OUT_F16 2
@@ -78,6 +85,12 @@ struct OutSpec {
     const float *a_scale;
     const float *b_scale;
     int type;
+    float beta;
+    const void *c;
+    int c_type;
+    const float *c_scale;
+    const float *d_scale;
+    float *amax;
 };
 
 __device__ __forceinline__ float out_scale(const OutSpec &o)
@@ -86,6 +99,22 @@ __device__ __forceinline__ float out_scale(const OutSpec &o)
     if (o.a_scale) s *= *o.a_scale;
     if (o.b_scale) s *= *o.b_scale;
     return s;
+}
+
+// the three factors of the epilogue, read once per kernel
+struct OutFactors {
+    float ab, c, d;
+};
+
+__device__ __forceinline__ OutFactors out_factors(const OutSpec &o)
+{
+    // (the same in every lane: pinned to scalar registers, the kernels are short of vector ones)
+    const auto uniform = [](float v) { return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v))); };
+    OutFactors f;
+    f.ab = uniform(out_scale(o));
+    f.c = uniform(o.c ? (o.c_scale ? o.beta * *o.c_scale : o.beta) : 0.0f);
+    f.d = uniform(o.d_scale ? *o.d_scale : 1.0f);
+    return f;
 }
 
 __device__ __forceinline__ uint32_t out_bits16(float v, int type)
@@ -130,6 +159,74 @@ __device__ __forceinline__ void store_out4(void *base, size_t index, v4f v, int 
         *(FP8GEMM_GLOBAL v4f *)((FP8GEMM_GLOBAL float *)base + index) = v;
     else
         *(FP8GEMM_GLOBAL v2u *)((FP8GEMM_GLOBAL unsigned short *)base + index) = out_pack4(v, type);
+}
+
+// element `index` of an input matrix of the given type (the C operand of the epilogue)
+__device__ __forceinline__ float load_in(const void *base, size_t index, int type)
+{
+    if (type == FP8GEMM_DEV_OUT_F32) return ((const FP8GEMM_GLOBAL float *)base)[index];
+    const unsigned short h = ((const FP8GEMM_GLOBAL unsigned short *)base)[index];
+    if (type == FP8GEMM_DEV_OUT_BF16) return __builtin_bit_cast(float, (uint32_t)h << 16);
+    return (float)__builtin_bit_cast(_Float16, h);
+}
+
+// four consecutive elements starting at `index` (index % 4 == 0, 16-byte aligned base)
+__device__ __forceinline__ v4f load_in4(const void *base, size_t index, int type)
+{
+    if (type == FP8GEMM_DEV_OUT_F32) return *(const FP8GEMM_GLOBAL v4f *)((const FP8GEMM_GLOBAL float *)base + index);
+    const v2u w = *(const FP8GEMM_GLOBAL v2u *)((const FP8GEMM_GLOBAL unsigned short *)base + index);
+    v4f r;
+    if (type == FP8GEMM_DEV_OUT_BF16) {
+        r[0] = __builtin_bit_cast(float, w[0] << 16);
+        r[1] = __builtin_bit_cast(float, w[0] & 0xFFFF0000u);
+        r[2] = __builtin_bit_cast(float, w[1] << 16);
+        r[3] = __builtin_bit_cast(float, w[1] & 0xFFFF0000u);
+    } else {
+        r[0] = (float)__builtin_bit_cast(_Float16, (unsigned short)(w[0] & 0xFFFFu));
+        r[1] = (float)__builtin_bit_cast(_Float16, (unsigned short)(w[0] >> 16));
+        r[2] = (float)__builtin_bit_cast(_Float16, (unsigned short)(w[1] & 0xFFFFu));
+        r[3] = (float)__builtin_bit_cast(_Float16, (unsigned short)(w[1] >> 16));
+    }
+    return r;
+}
+
+// The epilogue of one element / of four consecutive ones: fp32 sum -> value to store, and the
+// thread's running largest |y| (NaNs do not enter it).
+__device__ __forceinline__ float finish_one(const OutSpec &o, const OutFactors &f, size_t index, float sum, float &amax)
+{
+    float y = sum * f.ab;
+    if (o.c) y += f.c * load_in(o.c, index, o.c_type);
+    amax = fmaxf(amax, fabsf(y));
+    return y * f.d;
+}
+
+__device__ __forceinline__ v4f finish_four(const OutSpec &o, const OutFactors &f, size_t index, v4f sum, float &amax)
+{
+    v4f y = {sum[0] * f.ab, sum[1] * f.ab, sum[2] * f.ab, sum[3] * f.ab};
+    if (o.c) {
+        const v4f c = load_in4(o.c, index, o.c_type);
+        y[0] += f.c * c[0];
+        y[1] += f.c * c[1];
+        y[2] += f.c * c[2];
+        y[3] += f.c * c[3];
+    }
+    amax = fmaxf(fmaxf(amax, fmaxf(fabsf(y[0]), fabsf(y[1]))), fmaxf(fabsf(y[2]), fabsf(y[3])));
+    y[0] *= f.d;
+    y[1] *= f.d;
+    y[2] *= f.d;
+    y[3] *= f.d;
+    return y;
+}
+
+// Folds the threads' largest magnitudes into *o.amax (which the host has set to zero on the
+// stream before the kernel): one atomic per wave.  Non-negative floats order like their bit
+// patterns, so an integer maximum does it.
+__device__ __forceinline__ void amax_commit(const OutSpec &o, float amax)
+{
+    if (!o.amax) return;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    if ((threadIdx.x & 63) == 0 && amax > 0.0f) atomicMax(reinterpret_cast<int *>(o.amax), __builtin_bit_cast(int, amax));
 }
 
 // The same with the streaming (non-temporal) hint, for results that no kernel reads again:

@@ -115,9 +115,10 @@ hipError_t launch_ptile_work(const PtileWork &w, int m, int k, int n, const uint
                              float *ws, int rotate, const OutSpec &spec, hipStream_t stream)
 {
     auto kernel = gemm_ptile_kernel<S, AF, BF, KOVER, EX, BSTREAM>;
-    hipError_t e = allow_lds<PtileKernelTag<S, AF, BF, KOVER, EX, BSTREAM>>(kernel, S::PTILE_LDS_BYTES);
+    constexpr int kLdsBytes = S::PTILE_LDS_BYTES + 256;      // + the landing place of the L2 prefetches
+    hipError_t e = allow_lds<PtileKernelTag<S, AF, BF, KOVER, EX, BSTREAM>>(kernel, kLdsBytes);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * w.slots)), dim3(S::THREADS), S::PTILE_LDS_BYTES, stream,
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * w.slots)), dim3(S::THREADS), kLdsBytes, stream,
                        m, k, n, a, b, out, ws, w.tiles_m, w.tiles_n, w.GM, tile_column_block(w.tiles_n, m, n, k), w.bulk, w.tail,
                        w.nsplit, w.rounds, rotate, spec);
     return hipGetLastError();

@@ -79,6 +79,8 @@ hipError_t static_scratch_address(void **out)
 
 }  // namespace
 
+__global__ void fill_float_kernel(float *p, float v) { *p = v; }
+
 hipError_t Workspace::get(size_t need, void **out)
 {
     if (!pooled_) {
@@ -101,7 +103,7 @@ hipError_t Workspace::get(size_t need, void **out)
 hipError_t launch_reduce(const float *ws, void *out, size_t count, int nsplit, const OutSpec &spec, hipStream_t stream)
 {
     const bool vec = count % 4 == 0 &&
-                     ((reinterpret_cast<uintptr_t>(ws) | reinterpret_cast<uintptr_t>(out)) % 16) == 0;
+                     ((reinterpret_cast<uintptr_t>(ws) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(spec.c)) % 16) == 0;
     if (vec) {
         const size_t count4 = count / 4;
         hipLaunchKernelGGL(gemm_splitk_reduce4_kernel, dim3((unsigned)((count4 + 255) / 256)), dim3(256), 0, stream,
@@ -164,7 +166,8 @@ size_t ptile_scratch_bytes(const PtileWork &w, int bm, int bn)
 
 bool plain_output(const OutSpec &spec)
 {
-    return spec.type == FP8GEMM_DEV_OUT_F32 && spec.alpha == 1.0f && !spec.a_scale && !spec.b_scale;
+    return spec.type == FP8GEMM_DEV_OUT_F32 && spec.alpha == 1.0f && !spec.a_scale && !spec.b_scale && !spec.c &&
+           !spec.d_scale && !spec.amax;
 }
 
 bool p2h_ok(int k, int nsplit)
@@ -315,7 +318,7 @@ size_t tile_plan_scratch_bytes(int m, int n, const TilePlan &p)
 
 namespace {
 
-const OutSpec kPlainOut = {1.0f, nullptr, nullptr, FP8GEMM_DEV_OUT_F32};
+const OutSpec kPlainOut = {1.0f, nullptr, nullptr, FP8GEMM_DEV_OUT_F32, 0.0f, nullptr, FP8GEMM_DEV_OUT_F32, nullptr, nullptr, nullptr};
 
 int launch_checked(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt, void *out,
                    int stages, int algo, int variant, int nsplit, void *stream, const OutSpec &spec,
@@ -416,15 +419,34 @@ int fp8gemm_launch_tuned(int m, int k, int n, const void *a, int a_fmt, const vo
     return launch_pooled(m, k, n, a, a_fmt, b, b_fmt, out, 2, algo, variant, split_k, stream);
 }
 
+int fp8gemm_launch_epilogue(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
+                            void *d, int d_type, float alpha, float beta, const void *c, int c_type,
+                            const float *a_scale, const float *b_scale, const float *c_scale, const float *d_scale,
+                            float *amax_d, void *stream)
+{
+    const auto type_ok = [](int t) { return t == FP8GEMM_OUT_F32 || t == FP8GEMM_OUT_BF16 || t == FP8GEMM_OUT_F16; };
+    if (!type_ok(d_type) || (c && !type_ok(c_type))) return (int)hipErrorInvalidValue;
+    if (!(alpha == alpha) || !(beta == beta)) return (int)hipErrorInvalidValue;      // NaN
+    // in place (c == d) only with one element type: a thread then reads exactly the bytes it overwrites
+    if (c && c == d && c_type != d_type) return (int)hipErrorInvalidValue;
+    if (m <= 0 || k <= 0 || n <= 0 || !a || !b || !d) return (int)hipErrorInvalidValue;
+    if (amax_d) {
+        // the kernels fold |y| into *amax_d with an atomic maximum, starting from zero
+        (void)hipGetLastError();
+        hipLaunchKernelGGL(fill_float_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream), amax_d, 0.0f);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return (int)e;
+    }
+    const OutSpec spec = {alpha, a_scale, b_scale, d_type, beta, c, c ? c_type : FP8GEMM_OUT_F32, c_scale, d_scale, amax_d};
+    return launch_pooled(m, k, n, a, a_fmt, b, b_fmt, d, 2, FP8GEMM_ALGO_AUTO, -1, 0, stream, spec);
+}
+
 int fp8gemm_launch_ex(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
                       void *out, int out_type, float alpha, const float *a_scale, const float *b_scale,
                       void *stream)
 {
-    if (out_type != FP8GEMM_OUT_F32 && out_type != FP8GEMM_OUT_BF16 && out_type != FP8GEMM_OUT_F16)
-        return (int)hipErrorInvalidValue;
-    if (!(alpha == alpha)) return (int)hipErrorInvalidValue;      // NaN
-    const OutSpec spec = {alpha, a_scale, b_scale, out_type};
-    return launch_pooled(m, k, n, a, a_fmt, b, b_fmt, out, 2, FP8GEMM_ALGO_AUTO, -1, 0, stream, spec);
+    return fp8gemm_launch_epilogue(m, k, n, a, a_fmt, b, b_fmt, out, out_type, alpha, 0.0f, nullptr, FP8GEMM_OUT_F32,
+                                   a_scale, b_scale, nullptr, nullptr, nullptr, stream);
 }
 
 int fp8gemm_num_variants(int algo)

@@ -55,13 +55,18 @@ __global__ __launch_bounds__(64) void gemm_direct_kernel(int M, int K, int N,
     }
 
     const int col = n0 + i;
+    const OutFactors ofac = out_factors(spec);
+    float amax_local = 0.0f;
     if (col < N) {
-        const float scale = out_scale(spec);
         for (int r = 0; r < 16; ++r) {
             const int row = m0 + 8 * (r >> 2) + 4 * g + (r & 3);
-            if (row < M) store_out(C, (size_t)row * N + col, acc[r] * scale, spec.type);
+            if (row < M) {
+                const size_t index = (size_t)row * N + col;
+                store_out(C, index, finish_one(spec, ofac, index, acc[r], amax_local), spec.type);
+            }
         }
     }
+    amax_commit(spec, amax_local);
 }
 
 #endif  // FP8GEMM_KERNEL_DIRECT_H

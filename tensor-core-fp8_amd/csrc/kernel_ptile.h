@@ -51,8 +51,11 @@ __device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xC
 // in it across the statement; it warns that M0 is a reserved register, which is the point.
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
+// (lds_addr is the same in every lane; where the compiler has let it drift into a vector
+// register, v_readfirstlane_b32 brings it back -- otherwise the call is folded away)
 __device__ __forceinline__ void buffer_load_lds_b128(v4i rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff)
 {
+    lds_addr = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
                  : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
@@ -61,10 +64,20 @@ __device__ __forceinline__ void buffer_load_lds_b128(v4i rsrc, uint32_t lds_addr
 // the same with the non-temporal hint, for an operand that no other workgroup reads
 __device__ __forceinline__ void buffer_load_lds_b128_stream(v4i rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff)
 {
+    lds_addr = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen nt lds"
                  :
                  : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
                  : "m0");
+}
+// One 4-byte-per-lane load from per-lane addresses straight into LDS at lds_addr + lane*4.
+__device__ __forceinline__ void global_load_lds_b32(const uint8_t *ptr, uint32_t lds_addr)
+{
+    lds_addr = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
+                 :
+                 : "s"(lds_addr), "v"(ptr)
+                 : "m0", "memory");
 }
 #pragma clang diagnostic pop
 
@@ -161,12 +174,14 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
 
     // item of round r: tile, slice, K-tile range [kt0, kt0 + T), scratch slot (-1: writes C);
     // false when this workgroup has none
+    int items_in_xcd = 32;             // work items of this round on this workgroup's XCD
     auto tile_of_round = [&](int r, int &tm, int &tn, int &kt0, int &T, int &ws_slot) -> bool {
         if (r >= rounds) return false;
         int g, slice = 0;
         ws_slot = -1;
         if (r < bulk_rounds) {
             if (slot >= 32) return false;
+            items_in_xcd = 32;
             g = r * 256 + xcd * 32 + slot;
         } else {
             const int first = (r - bulk_rounds) * 256;
@@ -174,6 +189,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
             count = count > 256 ? 256 : count;
             if (count <= 0) return false;
             const int per_xcd = (count + 7) >> 3;
+            items_in_xcd = per_xcd;
             const int local = xcd * per_xcd + slot;
             if (slot >= per_xcd || local >= count) return false;
             const int u = first + local;
@@ -213,6 +229,33 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
     const uint32_t ldsA = lds_base + (uint32_t)(wave * S::A_LOADS * RPI * BK);
     const uint32_t ldsB = lds_base + (uint32_t)(BM * BK + wave * S::B_LOADS * RPI * BK);
     v4i rsA = {0, 0, 0, 0}, rsB = {0, 0, 0, 0};
+    // L2 prefetch: after the loads of a K tile each wave touches, with one 4-byte load per lane
+    // whose data nobody uses, one 128-byte line per lane of the K tile pf_dist further on, so
+    // that the line is on its way from HBM or the last-level cache into this XCD's L2 a K tile
+    // and more before the loads that need it (whose own latency budget is about one K tile).
+    // The workgroups of an XCD that share a panel split its rows among them, so that every line
+    // is asked for once per XCD: with strips of GM tile rows, GM workgroups share a panel of B
+    // and up to 8 share a panel of A.  B comes first (where C has one row of tiles it is
+    // the operand that streams from HBM), A takes the lanes that are left.
+    const uint8_t *pf_ptr = A;
+    auto plan_prefetch = [&](int tile_m_, int tile_n_, int items_in_xcd) __attribute__((always_inline)) {
+        const int q = wave * 64 + lane;                      // 0 .. 255: line number inside this workgroup's share
+        int a_parts = items_in_xcd / GM;
+        a_parts = a_parts > 8 ? 8 : (a_parts < 1 ? 1 : a_parts);
+        const int nb = (BN + GM - 1) / GM, na = (BM + a_parts - 1) / a_parts;
+        const int bpart = slot % GM, apart = (slot / GM) % a_parts;
+        const uint8_t *p = A + (size_t)(tile_m_ * BM) * K;   // lanes without a line of their own: one valid address
+        if (q < nb) {
+            int row = tile_n_ * BN + bpart * nb + q;
+            row = row < N ? row : N - 1;
+            p = B + (size_t)row * K;
+        } else if (q - nb < na) {
+            int row = tile_m_ * BM + apart * na + (q - nb);
+            row = row < M ? row : M - 1;
+            p = A + (size_t)row * K;
+        }
+        pf_ptr = p;
+    };
     // K walk of the planned item: K tiles kt_base + ((t + kt_rot) mod kt_count), t = 0, 1, ..
     // The rotation kt_rot only reorders the fp32 sum.  Workgroups that walk K in step read,
     // at any moment, addresses that agree in the bits below the row stride; with a
@@ -233,6 +276,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         const unsigned key = rotate == 1 ? (unsigned)tile_n : (unsigned)item;   // item: (round, XCD)
         // (the division runs on the vector unit; the result is the same in every lane)
         kt_rot = rotate == 0 ? 0 : __builtin_amdgcn_readfirstlane((int)(((key * 2654435761u) >> 8) % (unsigned)count));
+        plan_prefetch(tile_m, tile_n, items_in_xcd);
     };
     // load number j (0 .. LOADS-1) of step `ktile` of the planned item's K walk into ring slot `stage`
     // (the lambdas around the loads are forced inline: a closure left in memory would turn the
@@ -263,6 +307,26 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
 #pragma unroll
         for (int j = 0; j < S::LOADS; ++j) issue_load(j, ktile, stage);
     };
+
+    // (a load that writes LDS, into 256 bytes past everything else that nobody reads: a load
+    // into a register would write that register whenever it returns, behind the compiler's back)
+    auto issue_prefetch = [&](int ktile) __attribute__((always_inline)) {
+        if constexpr (BSTREAM) return;
+        int kk = ktile < kt_count ? ktile : kt_count - 1;
+        kk += kt_rot;
+        kk = kk >= kt_count ? kk - kt_count : kk;
+        // (K is a multiple of 16: the last, overhanging K tile still starts inside the row)
+        const uint32_t koff = (uint32_t)__builtin_amdgcn_readfirstlane((kt_base + kk) * BK);
+        global_load_lds_b32(pf_ptr + koff, lds_base + (uint32_t)S::PTILE_LDS_BYTES);
+    };
+    // Prefetch instructions that close a batch of loads, and how many K tiles they run ahead of
+    // the batch.  One K tile ahead is best (MI355X, 16384^3: 56.4 % of the FP8 peak without, 60.9 %
+    // one K tile ahead, 60.7 / 60.3 / 59.6 % two / three / four ahead; 3072^3 ... 6144^3 gain 1-3 %,
+    // shapes whose operands stay in the caches are unchanged).  Not where B streams past with the
+    // non-temporal hint (one row of tiles: M=256 N=28672 K=8192 76 -> 84 us with the prefetch):
+    // there every line is used once, by one workgroup, and asking for it twice only adds requests.
+    constexpr int NPF = BSTREAM ? 0 : 1;
+    constexpr int pf_dist = 1;
 
     int tile_m = 0, tile_n = 0, kt0 = 0, T = 0, ws_slot = -1;
     bool have = tile_of_round(0, tile_m, tile_n, kt0, T, ws_slot);
@@ -322,7 +386,10 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
             // with the loads (and may retire out of order with them), so wait for all.
             wait_vmcnt<0>();
             __syncthreads();
-            if (STAGES - 1 < T) issue_all_loads(STAGES - 1, STAGES - 1);
+            if (STAGES - 1 < T) {
+                issue_all_loads(STAGES - 1, STAGES - 1);
+                issue_prefetch(STAGES - 1 + pf_dist);
+            }
             using I0 = std::integral_constant<int, 0>;
             using I1 = std::integral_constant<int, 1>;
 #pragma unroll
@@ -347,9 +414,11 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                     if (next) {
                         // every fragment read of K tile t has been issued; once they have
                         // returned this wave no longer needs the ring slot
+                        // K tile t + 1 has landed once only the younger batches of loads (each
+                        // closed by its prefetch) and the prefetch that closed its own are left
                         wait_lgkmcnt0();
                         if (load)
-                            wait_vmcnt<S::LOADS *(STAGES - 2)>();
+                            wait_vmcnt<(S::LOADS + NPF) * (STAGES - 2) + NPF>();
                         else
                             wait_vmcnt<0>();
                         __syncthreads();
@@ -367,6 +436,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
 #pragma unroll
                         for (int u = 0; u < LD_PER; ++u)
                             if (m * LD_PER + u < S::LOADS) issue_load(m * LD_PER + u, t + STAGES, stage);
+                        if (m == NMFMA - 1) issue_prefetch(t + STAGES + pf_dist);
                     }
                     if (reads) {
 #pragma unroll
@@ -437,6 +507,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
             wait_vmcnt<0>();
             __syncthreads();
             if (1 < T) issue_all_loads(1, 1);
+            issue_prefetch(1 + pf_dist);
             read_a(0, 0, 0);
             read_a(0, 1, 0);
 
@@ -455,8 +526,10 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 if (next) {
+                    // every load but the youngest has landed: the youngest is the prefetch that
+                    // closed the previous batch of loads, whose data nobody waits for
                     wait_lgkmcnt0();
-                    wait_vmcnt<0>();
+                    wait_vmcnt<NPF>();
                     __syncthreads();
                 }
 #pragma unroll
@@ -473,6 +546,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                     } else if (next) {
                         read_b(PN{}, m >> 2, (m >> 1) & 1, nstage);
                     }
+                    if (m == 31 && load) issue_prefetch(t + 2 + pf_dist);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             };
@@ -522,10 +596,16 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         void *__restrict__ tile_base = to_ws ? static_cast<void *>(ws) : C;
         const size_t tile_origin = to_ws ? (size_t)ws_slot * (size_t)(BM * BN) : (size_t)m0 * (size_t)N + n0;
         const size_t ldo = to_ws ? (size_t)BN : (size_t)N;
-        const int otype = (!EX || to_ws) ? FP8GEMM_DEV_OUT_F32 : spec.type;
-        const float oscale = (!EX || to_ws) ? 1.0f : out_scale(spec);
+        // (the epilogue arithmetic -- scales, beta * C, largest magnitude -- only where C itself is
+        // written, and only in the kernels compiled for it)
+        const bool finish = EX && !to_ws;
+        const int otype = finish ? spec.type : FP8GEMM_DEV_OUT_F32;
+        OutFactors ofac = {1.0f, 0.0f, 1.0f};
+        if (finish) ofac = out_factors(spec);
+        float amax_local = 0.0f;
         const bool full = to_ws || ((m0 + BM <= M) && (n0 + BN <= N) && (N % 4 == 0) &&
-                                    (reinterpret_cast<uintptr_t>(C) % 16 == 0));
+                                    (reinterpret_cast<uintptr_t>(C) % 16 == 0) &&
+                                    (!EX || !spec.c || reinterpret_cast<uintptr_t>(spec.c) % 16 == 0));
         {
             // Each wave transposes its results through a private strip of LDS (the part of
             // the ring the next tile's first loads do not use, plus the LDS above the ring)
@@ -581,12 +661,14 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                     if constexpr (ST + 1 < NSTEP) stage_strip(std::integral_constant<int, ST + 1>{});
                     __builtin_amdgcn_sched_barrier(0);
                     if (EX) {
+                        if (finish) {
+                            // (four rows at a time: all the reads of C at once would need a second
+                            // set of registers as large as buf)
 #pragma unroll
-                        for (int u = 0; u < NR; ++u) {
-                            buf[u][0] *= oscale;
-                            buf[u][1] *= oscale;
-                            buf[u][2] *= oscale;
-                            buf[u][3] *= oscale;
+                            for (int u = 0; u < NR; ++u) {
+                                buf[u] = finish_four(spec, ofac, first + (size_t)(u * RPI_ST) * ldo, buf[u], amax_local);
+                                if ((u & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+                            }
                         }
                     }
                     // partial sums in the scratch are read back soon (keep them cached);
@@ -603,17 +685,14 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
 #pragma unroll 2
                     for (int r0 = 0; r0 < 32; r0 += RPI_ST) {
                         v4f v = *reinterpret_cast<const v4f *>(stg + (r0 + rl) * ROWB + cl * 16);
-                        if (EX) {
-                            v[0] *= oscale;
-                            v[1] *= oscale;
-                            v[2] *= oscale;
-                            v[3] *= oscale;
-                        }
                         const size_t index = first + (size_t)r0 * ldo;
                         if (m0 + lrow0 + r0 < M) {
 #pragma unroll
                             for (int e = 0; e < 4; ++e)
-                                if (n0 + lcol_ + e < N) store_out(tile_base, index + e, v[e], otype);
+                                if (n0 + lcol_ + e < N) {
+                                    const float y = (EX && finish) ? finish_one(spec, ofac, index + e, v[e], amax_local) : v[e];
+                                    store_out(tile_base, index + e, y, otype);
+                                }
                         }
                     }
                     if constexpr (ST + 1 < NSTEP) stage_strip(std::integral_constant<int, ST + 1>{});
@@ -621,6 +700,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
             };
             stage_strip(std::integral_constant<int, 0>{});
             static_for<0, NSTEP>(drain_strip);
+            if (EX && finish) amax_commit(spec, amax_local);
         }
         tile_m = next_m;
         tile_n = next_n;

@@ -180,9 +180,11 @@ __global__ __launch_bounds__(64) void gemm_skinny_kernel(int M, int K, int N,
     // with K slices `out` is the fp32 scratch (plane `split`, bare sums; the reduction
     // applies scale and output type), otherwise the output matrix itself
     const bool partial = nsplit > 1;
-    const float scale = partial ? 1.0f : out_scale(spec);
     const int type = partial ? FP8GEMM_DEV_OUT_F32 : spec.type;
     const size_t plane = partial ? (size_t)split * M * N : 0;
+    OutFactors ofac = {1.0f, 0.0f, 1.0f};
+    if (!partial) ofac = out_factors(spec);
+    float amax_local = 0.0f;
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
@@ -190,8 +192,13 @@ __global__ __launch_bounds__(64) void gemm_skinny_kernel(int M, int K, int N,
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int row = i * 16 + 4 * fq + r;
-                if (row < M) store_out(out, plane + (size_t)row * N + n0 + j * 16 + fi, acc[i][j][r] * scale, type);
+                if (row < M) {
+                    const size_t index = plane + (size_t)row * N + n0 + j * 16 + fi;
+                    const float y = partial ? acc[i][j][r] : finish_one(spec, ofac, index, acc[i][j][r], amax_local);
+                    store_out(out, index, y, type);
+                }
             }
+    if (!partial) amax_commit(spec, amax_local);
 }
 
 #endif  // FP8GEMM_KERNEL_SKINNY_H
