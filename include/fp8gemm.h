@@ -130,7 +130,7 @@ int fp8gemm_launch_algo(int m, int k, int n, const void *a, int a_fmt, const voi
  * and one of its compiled shape variants (0 .. fp8gemm_num_variants(algo)-1,
  * -1 = the default for the shape).  For FP8GEMM_ALGO_SKINNY, variant may add
  * 16 * columns-per-wave/16 to override the planned column count per wave; for
- * FP8GEMM_ALGO_TILE it may add 16 * (1 + r) to force the K-walk rotation mode
+ * FP8GEMM_ALGO_TILE it may add 32 * (1 + r) to force the K-walk rotation mode
  * r (0 none, 1 per tile column, 2 per XCD and round).  split_k > 0 overrides
  * the planned number of K slices (skinny kernel and persistent tiled kernels);
  * split_k < 0 (tiled kernels only) cuts only the tiles that do not fill a

@@ -32,6 +32,12 @@ using TileT2 = TileShape<192, 256, 128, 2, 2, 2, 3>;  // persistent, three-quart
 using TileT4 = TileShape<192, 256, 64, 2, 2, 4, 2>;
 using TileH4 = TileShape<128, 256, 64, 2, 2, 4, 2>;
 using TileQ4 = TileShape<128, 128, 64, 2, 2, 4, 2>;
+// weight streaming through the tiled kernel (one row of tiles, B read once with the non-temporal hint):
+// deep rings, so that many bytes of B are in flight per CU
+// (M=64 N=28672 K=8192, weights cold: 39.3 us against 50.0 us of the single-wave streaming kernel; rings of 4, 5
+// and 6 slots run alike, 64-byte K tiles in an 8-deep ring 57 us, a 64 x 256 tile 54 us)
+using TileE5 = TileShape<64, 128, 128, 1, 4, 5, 3>;    // up to 64 rows of A: four waves of 64 x 32, 5 x 24 KiB ring
+using TileQ4s = TileShape<128, 128, 128, 2, 2, 4, 3>;  // up to 128 rows: the quarter tile with a 4 x 32 KiB ring
 
 // Skinny kernel shapes: <MT, TN, BK, stages>.
 template <int MT, int TN>
@@ -202,6 +208,8 @@ hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, 
     case 14:
         if (!p2h_ok(k, nsplit)) return hipErrorInvalidValue;
         return launch_ptile_shape<TileT2h, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+    case 15: return launch_ptile_shape<TileE5, AF, BF, false, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+    case 16: return launch_ptile_shape<TileQ4s, AF, BF, false, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -279,11 +287,11 @@ hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, voi
         if (variant >= 0) {
             // tuning hook: variant = shape index + 16 * (1 + K-walk rotation mode); a bare
             // shape index keeps the plan's rotation and runs unsplit unless split_k says otherwise
-            if (variant >= 16) {
-                p.rotate = variant / 16 - 1;
+            if (variant >= 32) {
+                p.rotate = variant / 32 - 1;
                 if (p.rotate > 2) return hipErrorInvalidValue;
             }
-            p.variant = variant % 16;
+            p.variant = variant % 32;
             p.nsplit = 1;
             p.split_all = false;
         }

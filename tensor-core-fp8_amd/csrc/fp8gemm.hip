@@ -175,6 +175,7 @@ bool p2h_ok(int k, int nsplit)
     return k % 128 == 0 && (k / 128) / nsplit >= 2;
 }
 
+// the single-wave streams, up to 64 rows
 bool skinny_ok(int m, int k, int n)
 {
     return m <= 64 && n % 16 == 0 && k % 128 == 0;
@@ -214,9 +215,13 @@ SkinnyPlan plan_skinny(int m, int k, int n)
     return p;
 }
 
+// Up to 16 rows of A the single-wave streams are the fastest form (M=16 N=28672 K=8192: 37.0 us
+// against 38.0 us of the 64 x 128 tile); from 17 rows on the tiled kernel's deep shared ring
+// wins (M=32 38.5 against 40.5 us, M=64 39.3 against 50.0 us): a stream of its own per wave
+// re-reads all of A for every 64 columns.
 int select_algo(int m, int k, int n)
 {
-    if (skinny_ok(m, k, n)) return FP8GEMM_ALGO_SKINNY;
+    if (skinny_ok(m, k, n) && m <= 16) return FP8GEMM_ALGO_SKINNY;
     if (k % 16 == 0 && k <= (1 << 23)) return FP8GEMM_ALGO_TILE;
     return FP8GEMM_ALGO_DIRECT;
 }
@@ -247,6 +252,10 @@ constexpr PtileCost kPtileCosts[] = {
     {5, 11, 128, 256, 1.00, 6.0, 6.5e6},
     {6, 12, 128, 128, 0.75, 2.5, 4.0e6},
     {8, -1, 256, 128, 0.90, 10.0, 4.6e6},
+    // weight streaming (one row of tiles, B loaded once with the non-temporal hint, deep rings); their rings
+    // are 5 and 4 slots deep, so the 4-stage entry points run them too
+    {15, 15, 64, 128, 0.586, 5.5, 6.4e6},
+    {16, 16, 128, 128, 0.70, 5.5, 6.0e6},
 };
 constexpr double kIdleChipFactor = 0.6;
 constexpr int kSplitChoices[] = {1, 2, 3, 4, 6, 8, 12, 16};
@@ -262,6 +271,10 @@ TilePlan plan_tile(int m, int k, int n, int stages)
         // the 256 x 128 tile pays off where it holds all rows of A at once (no second
         // row of tiles re-reading the same B rows) and is at least half full
         if (c.variant == 8 && (m <= 128 || m > 256)) continue;
+        // the weight-streaming tiles: one row of tiles, whole 128-byte K tiles
+        if ((c.variant == 15 || c.variant == 16) && (m > c.bm || k % 128 != 0)) continue;
+        // ... and up to 64 rows nothing else comes close to them
+        if (m <= 64 && k % 128 == 0 && c.variant != 15) continue;
         if (stages == 4) {
             // the 4-deep rings rank like their 2- and 3-deep twins (same tiles, same work list);
             // only the 256 x 256 one is compiled for a K that is not a multiple of its K tile

@@ -56,7 +56,8 @@ def test_kernel_selection_is_pure_host_logic(pkg):
     assert L.fp8gemm_select_algo(8192, 8192, 8192) == pkg.ALGO_TILE
     assert L.fp8gemm_select_algo(16, 8192, 28672) == pkg.ALGO_SKINNY
     assert L.fp8gemm_select_algo(1, 28672, 8192) == pkg.ALGO_SKINNY
-    assert L.fp8gemm_select_algo(64, 8192, 10240) == pkg.ALGO_SKINNY
+    assert L.fp8gemm_select_algo(17, 8192, 10240) == pkg.ALGO_TILE       # from 17 rows on: the 64 x 128 streaming tile
+    assert L.fp8gemm_select_algo(64, 8192, 10240) == pkg.ALGO_TILE
     assert L.fp8gemm_select_algo(256, 8192, 28672) == pkg.ALGO_TILE
     assert L.fp8gemm_select_algo(100, 100, 100) == pkg.ALGO_DIRECT       # k not a multiple of 16
     assert L.fp8gemm_select_algo(100, 112, 100) == pkg.ALGO_TILE         # k a multiple of 16: the last K tile overhangs
@@ -80,7 +81,14 @@ def test_kernel_selection_is_pure_host_logic(pkg):
     for shape in [(256, 28672, 8192), (64, 28672, 8192), (300, 4096, 500), (8192, 8192, 8192), (7168, 7168, 7168)]:
         slices = pkg.plan(*shape)[2]
         assert (L.fp8gemm_scratch_bytes(*shape) > 0) == (slices > 1)
-    assert L.fp8gemm_scratch_bytes(64, 28672, 8192) == pkg.plan(64, 28672, 8192)[2] * 64 * 8192 * 4
+    # 64 rows: the 64 x 128 weight-streaming tile with a deep ring, K cut where the columns give too few tiles
+    assert pkg.plan(64, 8192, 28672)[:3] == (pkg.ALGO_TILE, 15, 1)
+    assert pkg.plan(64, 8192, 28672, stages=4)[:3] == (pkg.ALGO_TILE, 15, 1)         # its ring is 5 deep: both entry points
+    fam, var, slices, _ = pkg.plan(64, 28672, 8192)
+    assert (fam, var) == (pkg.ALGO_TILE, 15) and slices > 1
+    assert L.fp8gemm_scratch_bytes(64, 28672, 8192) == slices * (8192 // 128) * 64 * 128 * 4
+    assert pkg.plan(128, 8192, 28672)[:3] == (pkg.ALGO_TILE, 16, 1)
+    assert pkg.plan(16, 28672, 8192)[0] == pkg.ALGO_SKINNY
     # 28 x 28 tiles of 256 x 256: three rounds of whole tiles, the 16 left over cut into K slices
     fam, var, slices, mode = pkg.plan(7168, 7168, 7168)
     assert fam == pkg.ALGO_TILE and slices > 1 and mode >= 16

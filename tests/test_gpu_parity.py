@@ -14,7 +14,7 @@ from conftest import finite_codes, random_codes
 pytestmark = pytest.mark.gpu
 
 PAIRS = [(0, 0), (1, 1), (0, 1), (1, 0)]
-ALGOS = {"direct": 1, "tile": 2, "skinny": 3}
+ALGOS = {"auto": 0, "direct": 1, "tile": 2, "skinny": 3}
 
 
 def run_gpu(pkg, A, fa, B, fb, **kw):
@@ -99,6 +99,7 @@ def test_all_finite_codes(pkg, oracle, fa, fb, algo, shape):
 @pytest.mark.parametrize("algo,shape", [
     ("direct", (64, 2048, 96)), ("tile", (256, 2048, 256)), ("tile", (384, 4096, 640)),
     ("skinny", (16, 4096, 512)), ("skinny", (64, 2048, 256)), ("skinny", (1, 8192, 256)),
+    ("auto", (64, 4096, 1536)), ("auto", (33, 8192, 640)), ("auto", (17, 2048, 2048)), ("auto", (100, 4096, 1920)),
 ])
 def test_normal_inputs_within_fp32_reordering_bound(pkg, oracle, fa, fb, algo, shape):
     """4*N(0,1) inputs (the four-pairings workload) against the plain bound
@@ -112,8 +113,9 @@ def test_normal_inputs_within_fp32_reordering_bound(pkg, oracle, fa, fb, algo, s
 
 
 @pytest.mark.parametrize("fa,fb", PAIRS)
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12])
-@pytest.mark.parametrize("shape", [(256, 256, 256), (300, 512, 200), (1000, 1024, 900), (513, 384, 257), (64, 128, 2048)])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 15, 16])
+@pytest.mark.parametrize("shape", [(256, 256, 256), (300, 512, 200), (1000, 1024, 900), (513, 384, 257), (64, 128, 2048),
+                                   (40, 640, 1000)])
 def test_every_tile_variant(pkg, oracle, variant, shape, fa, fb):
     """Each compiled shape of the tiled kernels (persistent and one-tile-per-workgroup),
     on shapes that overhang the tile in m and n, for all four pairings."""
@@ -157,7 +159,8 @@ def test_16x16x128_variant_refuses_a_single_k_tile(pkg, variant):
         run_gpu(pkg, A, 0, B, 0, algo=ALGOS["tile"], variant=variant)
 
 
-@pytest.mark.parametrize("variant,split", [(0, 2), (0, 3), (1, 5), (5, 4), (5, 7), (6, 2), (6, 16), (2, 2), (8, 3), (13, 2), (13, 4), (14, 3)])
+@pytest.mark.parametrize("variant,split", [(0, 2), (0, 3), (1, 5), (5, 4), (5, 7), (6, 2), (6, 16), (2, 2), (8, 3), (13, 2), (13, 4), (14, 3),
+                                           (15, 3), (15, 4), (16, 2)])
 @pytest.mark.parametrize("shape", [(256, 2048, 512), (300, 4096, 200), (1000, 2304, 900), (128, 8192, 2048)])
 def test_tile_k_slices(pkg, oracle, variant, split, shape):
     """Persistent tiled kernels with the K range cut into slices whose partial sums are
@@ -287,7 +290,8 @@ def test_decode_through_mfma_is_bit_exact(pkg, oracle, fa, fb, algo):
     assert np.array_equal(C2, oracle.decode(A2, fa)[:, kn])
 
 
-@pytest.mark.parametrize("algo,variant", [("tile", 13), ("tile", 14), ("tile", 5), ("tile", 6), ("tile", 8), ("tile", 1)])
+@pytest.mark.parametrize("algo,variant", [("tile", 13), ("tile", 14), ("tile", 5), ("tile", 6), ("tile", 8), ("tile", 1), ("tile", 15),
+                                          ("tile", 16)])
 @pytest.mark.parametrize("fa,fb", PAIRS)
 def test_decode_through_mfma_every_persistent_form(pkg, oracle, fa, fb, algo, variant):
     """The same bit-exact selection test for the persistent tile shapes the planner uses
