@@ -194,6 +194,14 @@ size_t fp8gemm_scratch_held_bytes(void);
 int fp8gemm_launch_ws(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
                       float *out, int stages, void *workspace, size_t workspace_bytes, void *stream);
 
+/*
+ * The current device against what the plans are laid out for (MI355X as one partition: 256 CUs
+ * in 8 XCDs): info[0] = CUs of the device, info[1] = CUs the plans assume, info[2] = 1 on gfx950,
+ * info[3] = 1 when both match.  On any other layout the results are unchanged, only the plans
+ * are not tuned for it.  Returns 0 or a HIP error.
+ */
+int fp8gemm_device_info(int info[4]);
+
 /* Text for a return code (hipGetErrorString). */
 const char *fp8gemm_error_string(int code);
 

@@ -91,6 +91,8 @@ def lib():
     L.fp8gemm_plan.argtypes = [ci, ci, ci, ci, ctypes.POINTER(ci)]
     L.fp8gemm_scratch_bytes.restype = ctypes.c_size_t
     L.fp8gemm_scratch_bytes.argtypes = [ci, ci, ci]
+    L.fp8gemm_device_info.restype = ci
+    L.fp8gemm_device_info.argtypes = [ctypes.POINTER(ci)]
     L.fp8gemm_error_string.restype = ctypes.c_char_p
     L.fp8gemm_error_string.argtypes = [ci]
     L.fp8gemm_version.restype = ci

@@ -9,6 +9,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstring>
 #include <mutex>
 #include <utility>
 
@@ -28,7 +29,12 @@ extern template hipError_t dispatch<1, 1>(int, int, int, const uint8_t *, const 
                                           const OutSpec &, Workspace &, hipStream_t);
 
 namespace {
-constexpr int kVersion = 101;
+constexpr int kVersion = 102;
+// What the work lists and the planner's constants are laid out for: MI355X as one partition,
+// 256 CUs in 8 XCDs of 32, workgroups handed to the XCDs round robin (id mod 8).  On another
+// partition mode every result is still right (the work list only decides who computes what);
+// the plans are then merely not the best ones.  fp8gemm_device_info tells a caller which it is.
+constexpr int kPlannedCus = 256;
 constexpr int kMaxDevices = 64;
 
 // ------------------------------------------------------------------ scratch
@@ -398,6 +404,23 @@ int fp8gemm_launch_noalloc(int m, int k, int n, const void *a, int a_fmt, const 
     if (e != hipSuccess) return (int)e;
     Workspace wsp = Workspace::fixed(ptr, kStaticScratchBytes);
     return launch_checked(m, k, n, a, a_fmt, b, b_fmt, out, stages, FP8GEMM_ALGO_AUTO, -1, 0, stream, kPlainOut, wsp);
+}
+
+int fp8gemm_device_info(int info[4])
+{
+    if (!info) return (int)hipErrorInvalidValue;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess) return (int)e;
+    const bool gfx950 = std::strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+    info[0] = prop.multiProcessorCount;
+    info[1] = kPlannedCus;
+    info[2] = gfx950 ? 1 : 0;
+    info[3] = (gfx950 && prop.multiProcessorCount == kPlannedCus) ? 1 : 0;
+    return 0;
 }
 
 int fp8gemm_release_scratch(void)

@@ -124,8 +124,10 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                                                                  float *__restrict__ ws,
                                                                  int tiles_m, int tiles_n, int GM, int CB,
                                                                  int bulk, int tail, int nsplit,
-                                                                 int rounds, int rotate, OutSpec spec)
+                                                                 int rounds, int rotate_and_skew, OutSpec spec)
 {
+    const int rotate = rotate_and_skew & 0xFF;
+    const int skew = rotate_and_skew >> 8;
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, CH = S::CH, RPI = S::RPI;
     constexpr int STAGES = S::STAGES, TM = S::TM, TN = S::TN, KSTEPS = S::KSTEPS;
     constexpr int NMFMA = TM * TN;
@@ -327,6 +329,15 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
     // there every line is used once, by one workgroup, and asking for it twice only adds requests.
     constexpr int NPF = BSTREAM ? 0 : 1;
     constexpr int pf_dist = 1;
+
+    // Start skew: the workgroups of an XCD that work on tile row i of its window start i * skew
+    // ticks (10 ns each) late and stay that far apart for the rest of the launch, so that
+    // their epilogues -- which share the XCD's write path -- do not all come at once.
+    if (skew > 0 && bulk > 0) {
+        const unsigned long long ticks = (unsigned long long)((slot % GM) * skew);
+        const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();
+        while (__builtin_amdgcn_s_memrealtime() - t0 < ticks) __builtin_amdgcn_s_sleep(8);
+    }
 
     int tile_m = 0, tile_n = 0, kt0 = 0, T = 0, ws_slot = -1;
     bool have = tile_of_round(0, tile_m, tile_n, kt0, T, ws_slot);

@@ -159,3 +159,11 @@ def test_c_beyond_2_31_elements(pkg, oracle):
     out, dA, dB = gpu_gemm(pkg, A, 1, B, 0)
     rows = np.concatenate([np.arange(0, M, 997), np.arange(M - 40, M)]).astype(np.int32)
     check_rows(oracle, out, A, 1, B, 0, rows)      # the bound itself; K is short, so no margin is asked for
+
+
+def test_device_is_the_layout_the_plans_assume(pkg):
+    """MI355X as one partition: 256 CUs, gfx950 (the work lists number workgroups by XCD = id mod 8)."""
+    import ctypes
+    info = (ctypes.c_int * 4)()
+    assert pkg.lib().fp8gemm_device_info(info) == 0
+    assert list(info) == [256, 256, 1, 1]
