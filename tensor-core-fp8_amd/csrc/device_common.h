@@ -245,4 +245,30 @@ __device__ __forceinline__ void store_out4_stream(void *base, size_t index, v4f 
     }
 }
 
+// ---- device-scope accesses ---------------------------------------------------------------
+// The eight XCDs each have an L2 of their own, and a plain store may sit in the writer's L2
+// where a workgroup on another XCD does not see it.  Accesses with the sc1 bit act at device
+// scope: such a store is written through to memory before it counts as done (vmcnt), such a
+// load does not take a line that another XCD may have changed from its own L2.  Data handed
+// from one workgroup to another inside a launch goes through these, with the writer's
+// s_waitcnt vmcnt(0) and a device-scope atomic in between; no whole-cache write-back or
+// invalidate is needed.  (Buffer instructions, because their cache bits can be set from C++.)
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+constexpr int kDeviceScope = 16;      // the sc1 bit of a buffer instruction's cache policy
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t device_scope_window(void *base, uint32_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(base, 0, (int)bytes, 0x00020000);      // raw 32-bit data format
+}
+
+__device__ __forceinline__ void store_f32x4_device_scope(__amdgpu_buffer_rsrc_t window, uint32_t byte_offset, v4f v)
+{
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), window, (int)byte_offset, 0, kDeviceScope);
+}
+
+__device__ __forceinline__ v4f load_f32x4_device_scope(__amdgpu_buffer_rsrc_t window, uint32_t byte_offset)
+{
+    return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(window, (int)byte_offset, 0, kDeviceScope));
+}
+
 #endif  // FP8GEMM_DEVICE_COMMON_H

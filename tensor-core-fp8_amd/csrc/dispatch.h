@@ -38,6 +38,7 @@ using TileQ4 = TileShape<128, 128, 64, 2, 2, 4, 2>;
 // and 6 slots run alike, 64-byte K tiles in an 8-deep ring 57 us, a 64 x 256 tile 54 us)
 using TileE5 = TileShape<64, 128, 128, 1, 4, 5, 3>;    // up to 64 rows of A: four waves of 64 x 32, 5 x 24 KiB ring
 using TileQ4s = TileShape<128, 128, 128, 2, 2, 4, 3>;  // up to 128 rows: the quarter tile with a 4 x 32 KiB ring
+using TileW6 = TileShape<256, 128, 64, 2, 2, 6, 2>;    // half-width tile, 6 x 24 KiB ring
 
 // Skinny kernel shapes: <MT, TN, BK, stages>.
 template <int MT, int TN>
@@ -126,14 +127,14 @@ inline int start_skew(const PtileWork &w)
 // partial sums go through the scratch buffer and a reduction pass
 template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM>
 hipError_t launch_ptile_work(const PtileWork &w, int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
-                             float *ws, int rotate, const OutSpec &spec, hipStream_t stream)
+                             float *ws, int *counters, int rotate, const OutSpec &spec, hipStream_t stream)
 {
     auto kernel = gemm_ptile_kernel<S, AF, BF, KOVER, EX, BSTREAM>;
-    constexpr int kLdsBytes = S::PTILE_LDS_BYTES + 256;      // + the landing place of the L2 prefetches
+    constexpr int kLdsBytes = S::PTILE_LDS_BYTES + 256 + 16;      // + the landing place of the L2 prefetches + a flag
     hipError_t e = allow_lds<PtileKernelTag<S, AF, BF, KOVER, EX, BSTREAM>>(kernel, kLdsBytes);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * w.slots)), dim3(S::THREADS), kLdsBytes, stream,
-                       m, k, n, a, b, out, ws, w.tiles_m, w.tiles_n, w.GM, tile_column_block(w.tiles_n, m, n, k), w.bulk, w.tail,
+                       m, k, n, a, b, out, ws, counters, w.tiles_m, w.tiles_n, w.GM, tile_column_block(w.tiles_n, m, n, k), w.bulk, w.tail,
                        w.nsplit, w.rounds, rotate | (start_skew(w) << 8), spec);
     return hipGetLastError();
 }
@@ -147,22 +148,32 @@ hipError_t launch_ptile_shape_k(int m, int k, int n, const uint8_t *a, const uin
     if (k % 16 != 0 || k > (1 << 23) || nsplit < 1 || nsplit > (k + S::BK - 1) / S::BK) return hipErrorInvalidValue;
     const PtileWork w = ptile_work(m, n, S::BM, S::BN, nsplit, split_all);
     if (!w.ok) return hipErrorInvalidValue;
-    float *ws = nullptr;
+    // Scratch of a K-sliced launch: arrival counters, then the partial sums.  For tiles up to
+    // 128 x 128, where the counters can be relied on (see Workspace), the slice of a tile that
+    // arrives last adds the slices up inside the kernel; otherwise a reduction kernel follows.
+    // (One CU adding up four slices of a 256 x 256 tile reads 1 MiB: measured 6 to 15 us slower
+    // than the reduction kernel, which spreads that over the chip; for a 64 x 128 tile it is 128 KiB
+    // and 1 to 2 us faster than a second launch.)
+    constexpr bool kSumInKernel = ptile_sums_slices_in_kernel<S>;
+    float *base = nullptr, *ws = nullptr;
+    int *counters = nullptr;
     if (w.nsplit > 1) {
         void *p = nullptr;
         hipError_t e = wsp.get(ptile_scratch_bytes(w, S::BM, S::BN), &p);
         if (e != hipSuccess) return e;
-        ws = static_cast<float *>(p);
+        base = static_cast<float *>(p);
+        ws = base + kSliceCounterBytes / sizeof(float);
+        if (kSumInKernel && wsp.counters_zero() && w.tail <= kMaxSliceCounters) counters = static_cast<int *>(p);
     }
     hipError_t e;
     if constexpr (STREAM_TOO && !KOVER) {
-        e = w.tiles_m == 1 ? launch_ptile_work<S, AF, BF, KOVER, EX, true>(w, m, k, n, a, b, out, ws, rotate, spec, stream)
-                           : launch_ptile_work<S, AF, BF, KOVER, EX, false>(w, m, k, n, a, b, out, ws, rotate, spec, stream);
+        e = w.tiles_m == 1 ? launch_ptile_work<S, AF, BF, KOVER, EX, true>(w, m, k, n, a, b, out, ws, counters, rotate, spec, stream)
+                           : launch_ptile_work<S, AF, BF, KOVER, EX, false>(w, m, k, n, a, b, out, ws, counters, rotate, spec, stream);
     } else {
-        e = launch_ptile_work<S, AF, BF, KOVER, EX, false>(w, m, k, n, a, b, out, ws, rotate, spec, stream);
+        e = launch_ptile_work<S, AF, BF, KOVER, EX, false>(w, m, k, n, a, b, out, ws, counters, rotate, spec, stream);
     }
-    if (e != hipSuccess || w.nsplit == 1) return e;
-    return launch_tile_slices_reduce(ws, out, m, n, k, S::BM, S::BN, w, spec, stream);
+    if (e != hipSuccess || w.nsplit == 1 || counters) return e;
+    return launch_tile_slices_reduce(base, out, m, n, k, S::BM, S::BN, w, spec, stream);
 }
 
 // OVERHANG_TOO: this shape is also compiled for a K that is not a multiple of its K tile.
@@ -218,6 +229,7 @@ hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, 
         return launch_ptile_shape<TileT2h, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
     case 15: return launch_ptile_shape<TileE5, AF, BF, false, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
     case 16: return launch_ptile_shape<TileQ4s, AF, BF, false, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+    case 17: return launch_ptile_shape<TileW6, AF, BF, false, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -234,9 +246,10 @@ hipError_t launch_skinny_shape(int m, int k, int n, const uint8_t *a, const uint
     void *dst = out;
     if (nsplit > 1) {
         void *ws = nullptr;
-        hipError_t e = wsp.get((size_t)nsplit * m * n * sizeof(float), &ws);
+        // (the start of every scratch buffer belongs to the tiled kernel's arrival counters)
+        hipError_t e = wsp.get(kSliceCounterBytes + (size_t)nsplit * m * n * sizeof(float), &ws);
         if (e != hipSuccess) return e;
-        dst = ws;
+        dst = static_cast<unsigned char *>(ws) + kSliceCounterBytes;
     }
     auto kernel = gemm_skinny_kernel<S, AF, BF>;
     hipError_t e = allow_lds<SkinnyKernelTag<S, AF, BF>>(kernel, S::LDS_BYTES);

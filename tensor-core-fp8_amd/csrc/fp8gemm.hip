@@ -41,7 +41,15 @@ constexpr int kMaxDevices = 64;
 // Device runtime behind the scratch bookkeeping (scratch_pool.h).
 struct HipScratchBackend {
     using Event = hipEvent_t;
-    int alloc(size_t bytes, void **ptr) { return (int)hipMalloc(ptr, bytes); }
+    // (a new buffer starts with zeroed arrival counters; the kernels leave them at zero)
+    int alloc(size_t bytes, void **ptr)
+    {
+        hipError_t e = hipMalloc(ptr, bytes);
+        if (e != hipSuccess) return (int)e;
+        e = hipMemset(*ptr, 0, bytes < kSliceCounterBytes ? bytes : kSliceCounterBytes);
+        if (e != hipSuccess) (void)hipFree(*ptr);
+        return (int)e;
+    }
     void free(void *ptr) { (void)hipFree(ptr); }
     int record(void *stream, Event *ev)
     {
@@ -124,6 +132,7 @@ hipError_t launch_reduce(const float *ws, void *out, size_t count, int nsplit, c
 hipError_t launch_tile_slices_reduce(const float *ws, void *out, int m, int n, int k, int bm, int bn, const PtileWork &w,
                                      const OutSpec &spec, hipStream_t stream)
 {
+    ws += kSliceCounterBytes / sizeof(float);      // the partial sums follow the arrival counters
     const size_t threads = (size_t)w.tail * ((size_t)bm * bn / 4);
     hipLaunchKernelGGL(gemm_tile_slices_reduce_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream,
                        ws, out, m, n, bm, bn, w.tiles_m, w.tiles_n, w.GM, tile_column_block(w.tiles_n, m, n, k), w.bulk, w.tail,
@@ -167,7 +176,7 @@ int tile_column_block(int tiles_n, int m, int n, int k)
 
 size_t ptile_scratch_bytes(const PtileWork &w, int bm, int bn)
 {
-    return w.nsplit > 1 ? (size_t)w.nsplit * w.tail * bm * bn * sizeof(float) : 0;
+    return w.nsplit > 1 ? kSliceCounterBytes + (size_t)w.nsplit * w.tail * bm * bn * sizeof(float) : 0;
 }
 
 bool plain_output(const OutSpec &spec)
@@ -392,7 +401,7 @@ int fp8gemm_launch_ws(int m, int k, int n, const void *a, int a_fmt, const void 
                       float *out, int stages, void *workspace, size_t workspace_bytes, void *stream)
 {
     if (workspace && reinterpret_cast<uintptr_t>(workspace) % 16 != 0) return (int)hipErrorInvalidValue;
-    Workspace wsp = Workspace::fixed(workspace, workspace ? workspace_bytes : 0);
+    Workspace wsp = Workspace::fixed(workspace, workspace ? workspace_bytes : 0, false);
     return launch_checked(m, k, n, a, a_fmt, b, b_fmt, out, stages, FP8GEMM_ALGO_AUTO, -1, 0, stream, kPlainOut, wsp);
 }
 
@@ -402,7 +411,7 @@ int fp8gemm_launch_noalloc(int m, int k, int n, const void *a, int a_fmt, const 
     void *ptr = nullptr;
     const hipError_t e = static_scratch_address(&ptr);
     if (e != hipSuccess) return (int)e;
-    Workspace wsp = Workspace::fixed(ptr, kStaticScratchBytes);
+    Workspace wsp = Workspace::fixed(ptr, kStaticScratchBytes, true);      // static storage starts as zeros
     return launch_checked(m, k, n, a, a_fmt, b, b_fmt, out, stages, FP8GEMM_ALGO_AUTO, -1, 0, stream, kPlainOut, wsp);
 }
 
@@ -536,7 +545,7 @@ size_t fp8gemm_scratch_bytes(int m, int k, int n)
     const int algo = select_algo(m, k, n);
     if (algo == FP8GEMM_ALGO_SKINNY) nsplit = plan_skinny(m, k, n).nsplit;
     if (algo == FP8GEMM_ALGO_TILE) return tile_plan_scratch_bytes(m, n, plan_tile(m, k, n, 2));
-    return nsplit > 1 ? (size_t)nsplit * m * n * sizeof(float) : 0;
+    return nsplit > 1 ? kSliceCounterBytes + (size_t)nsplit * m * n * sizeof(float) : 0;
 }
 
 const char *fp8gemm_error_string(int code)

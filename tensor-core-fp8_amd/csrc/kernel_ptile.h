@@ -111,6 +111,11 @@ __device__ __forceinline__ v4i make_buffer_resource(const void *base, unsigned l
     return r;
 }
 
+// Whether the kernel for tile shape S can add up the K slices of a tile itself (the slice that
+// arrives last does it).  One CU then reads every slice of the tile, which pays up to 128 x 128.
+template <class S>
+constexpr bool ptile_sums_slices_in_kernel = S::BM * S::BN <= 128 * 128;
+
 // KOVER: the last K tile may overhang K (K % BK != 0); compiled separately so that the
 // common case carries no test for it.  EX: the output goes through `spec` (scale, fp32 /
 // bf16 / fp16); without it C receives the bare fp32 sums and `spec` is ignored.  BSTREAM: B is
@@ -122,6 +127,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                                                                  const uint8_t *__restrict__ B,
                                                                  void *__restrict__ C,
                                                                  float *__restrict__ ws,
+                                                                 int *__restrict__ counters,
                                                                  int tiles_m, int tiles_n, int GM, int CB,
                                                                  int bulk, int tail, int nsplit,
                                                                  int rounds, int rotate_and_skew, OutSpec spec)
@@ -131,6 +137,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, CH = S::CH, RPI = S::RPI;
     constexpr int STAGES = S::STAGES, TM = S::TM, TN = S::TN, KSTEPS = S::KSTEPS;
     constexpr int NMFMA = TM * TN;
+    constexpr bool SUM_HERE = ptile_sums_slices_in_kernel<S>;
     constexpr int NREADS = 2 * (TM + TN);          // ds_read_b128 per K step
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(LDS_AS uint8_t *)lds;
@@ -155,6 +162,9 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
     const uint32_t a_base = (uint32_t)(wm * (BM / S::WM) + fi) * BK;
     const uint32_t b_base = (uint32_t)(BM * BK) + (uint32_t)(wn * (BN / S::WN) + fi) * BK;
     const int KT = (K + BK - 1) / BK;              // K tiles of the whole problem; the last may overhang K
+    // the partial sums of the K slices, as a window for device-scope accesses (used with counters)
+    const __amdgpu_buffer_rsrc_t ws_window =
+        device_scope_window(ws, counters ? (uint32_t)nsplit * (uint32_t)tail * (uint32_t)(BM * BN * 4) : 0u);
 
     // Work items.  The tiles of C are numbered along strips of GM tile rows (down a
     // column of the strip first, then on to the next column), so that consecutive tile
@@ -684,7 +694,12 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                     }
                     // partial sums in the scratch are read back soon (keep them cached);
                     // C itself is not (streaming stores)
-                    if (to_ws) {
+                    if (SUM_HERE && to_ws && counters) {
+                        // (read back by a workgroup that may sit on another XCD)
+#pragma unroll
+                        for (int u = 0; u < NR; ++u)
+                            store_f32x4_device_scope(ws_window, (uint32_t)(first + (size_t)(u * RPI_ST) * ldo) * 4u, buf[u]);
+                    } else if (to_ws) {
 #pragma unroll
                         for (int u = 0; u < NR; ++u) store_out4(tile_base, first + (size_t)(u * RPI_ST) * ldo, buf[u], otype);
                     } else {
@@ -712,6 +727,75 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
             stage_strip(std::integral_constant<int, 0>{});
             static_for<0, NSTEP>(drain_strip);
             if (EX && finish) amax_commit(spec, amax_local);
+        }
+        // ---- K slices: the slice that arrives last adds them up ---------------------
+        // Every slice of a cut tile has written its partial sums to its scratch slot with
+        // device-scope stores.  Once those are done (the barrier waits for them) it counts
+        // itself on the tile's arrival counter, and the one that finds all the others there
+        // reads the slots back in slice order -- the order the reduction kernel uses, so the
+        // bits are the same -- and writes the tile of C.  Nobody waits for anybody.  The
+        // counter is left at zero for the next launch.
+        if (SUM_HERE && to_ws && counters) {                       // (uniform)
+            const int t_cut = ws_slot % tail;                      // number of the cut tile
+            LDS_AS int *flag = (LDS_AS int *)(lds + S::PTILE_LDS_BYTES + 256);
+            __syncthreads();                                       // (s_waitcnt vmcnt(0) ahead of the barrier)
+            if (tid == 0) {
+                const int before = __hip_atomic_fetch_add(counters + t_cut, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const int last = before == nsplit - 1;
+                if (last) __hip_atomic_store(counters + t_cut, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                *flag = last;
+            }
+            __syncthreads();
+            if (*flag) {
+                const uint32_t slot0 = (uint32_t)t_cut * (uint32_t)(BM * BN * 4);      // bytes
+                const uint32_t plane = (uint32_t)tail * (uint32_t)(BM * BN * 4);
+                OutFactors rfac = {1.0f, 0.0f, 1.0f};
+                if (EX) rfac = out_factors(spec);
+                float ramax = 0.0f;
+                const bool aligned = N % 4 == 0 && reinterpret_cast<uintptr_t>(C) % 16 == 0 &&
+                                     (!EX || !spec.c || reinterpret_cast<uintptr_t>(spec.c) % 16 == 0);
+                const int rtype = EX ? spec.type : FP8GEMM_DEV_OUT_F32;
+                constexpr int QUADS = BM * BN / 4;                 // groups of four columns in a tile
+                constexpr int QB = 4;                              // groups a thread has in flight
+                static_assert(QUADS % (S::THREADS * QB) == 0, "tile does not divide among the threads");
+                for (int q0 = tid; q0 < QUADS; q0 += S::THREADS * QB) {
+                    v4f sum[QB];
+#pragma unroll
+                    for (int u = 0; u < QB; ++u) sum[u] = load_f32x4_device_scope(ws_window, slot0 + (uint32_t)(q0 + u * S::THREADS) * 16u);
+                    for (int p = 1; p < nsplit; p += 2) {          // two more slices at a time
+                        const bool two = p + 1 < nsplit;
+                        v4f v0[QB], v1[QB];
+#pragma unroll
+                        for (int u = 0; u < QB; ++u) {
+                            const uint32_t at = slot0 + (uint32_t)(q0 + u * S::THREADS) * 16u + (uint32_t)p * plane;
+                            v0[u] = load_f32x4_device_scope(ws_window, at);
+                            if (two) v1[u] = load_f32x4_device_scope(ws_window, at + plane);
+                        }
+#pragma unroll
+                        for (int u = 0; u < QB; ++u) {
+                            sum[u] += v0[u];
+                            if (two) sum[u] += v1[u];
+                        }
+                    }
+#pragma unroll
+                    for (int u = 0; u < QB; ++u) {
+                        const int q = q0 + u * S::THREADS;
+                        const int row = q / (BN / 4), col = (q - row * (BN / 4)) * 4;
+                        const int grow = m0 + row, gcol = n0 + col;
+                        if (grow < M && gcol < N) {
+                            const size_t index = (size_t)grow * N + gcol;
+                            if (gcol + 3 < N && aligned) {
+                                store_out4_stream(C, index, EX ? finish_four(spec, rfac, index, sum[u], ramax) : sum[u], rtype);
+                            } else {
+                                for (int e = 0; e < 4; ++e)
+                                    if (gcol + e < N)
+                                        store_out(C, index + e, EX ? finish_one(spec, rfac, index + e, sum[u][e], ramax) : sum[u][e], rtype);
+                            }
+                        }
+                    }
+                }
+                if (EX) amax_commit(spec, ramax);
+            }
         }
         tile_m = next_m;
         tile_n = next_n;

@@ -16,7 +16,7 @@ namespace fp8gemm_detail {
 
 // tiled kernel shapes: 0 P2, 1 P4, 2 P8, 3 S2, 4 S4, 5 H3, 6 Q2, 7 S64, 8 W3, 9 T2, 10 T4, 11 H4, 12 Q4, 13 P2h, 14 T2h,
 // 15 E5, 16 Q4s
-constexpr int kNumTileVariants = 17;
+constexpr int kNumTileVariants = 18;
 constexpr int kNumSkinnyVariants = 6;
 
 // Work list of the persistent kernel for a tile shape: `bulk` tiles (a multiple of 256)
@@ -28,6 +28,10 @@ struct PtileWork {
     bool ok;
 };
 PtileWork ptile_work(int m, int n, int bm, int bn, int nsplit, bool split_all);
+// The scratch of a K-sliced launch starts with one arrival counter per cut tile (the slice that
+// arrives last adds the slices up), then the slices' partial sums follow.
+constexpr size_t kSliceCounterBytes = 16 * 1024;
+constexpr int kMaxSliceCounters = (int)(kSliceCounterBytes / sizeof(int));
 int tile_column_block(int tiles_n, int m, int n, int k);
 size_t ptile_scratch_bytes(const PtileWork &w, int bm, int bn);
 
@@ -58,17 +62,23 @@ size_t tile_plan_scratch_bytes(int m, int n, const TilePlan &p);
 // until the call's kernels are enqueued.
 class Workspace {
 public:
-    static Workspace pooled(hipStream_t stream) { return Workspace(stream, nullptr, 0, true); }
-    static Workspace fixed(void *ptr, size_t bytes) { return Workspace(nullptr, ptr, bytes, false); }
+    static Workspace pooled(hipStream_t stream) { return Workspace(stream, nullptr, 0, true, true); }
+    // counters_zero: the first kSliceCounterBytes of the buffer are known to hold zeros
+    static Workspace fixed(void *ptr, size_t bytes, bool counters_zero) { return Workspace(nullptr, ptr, bytes, false, counters_zero); }
     hipError_t get(size_t need, void **out);
+    // whether the arrival counters at the start of the buffer can be relied on (they start at
+    // zero and every kernel leaves them at zero): the pool's buffers and the static array, not a
+    // caller's workspace
+    bool counters_zero() const { return counters_zero_; }
 
 private:
-    Workspace(hipStream_t stream, void *ptr, size_t bytes, bool pooled)
-        : stream_(stream), ptr_(ptr), bytes_(bytes), pooled_(pooled) {}
+    Workspace(hipStream_t stream, void *ptr, size_t bytes, bool pooled, bool counters_zero)
+        : stream_(stream), ptr_(ptr), bytes_(bytes), pooled_(pooled), counters_zero_(counters_zero) {}
     hipStream_t stream_;
     void *ptr_;
     size_t bytes_;
     bool pooled_;
+    bool counters_zero_;
     std::unique_lock<std::mutex> lock_;
 };
 

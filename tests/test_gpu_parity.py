@@ -479,6 +479,36 @@ def test_caller_provided_workspace(pkg, oracle):
             assert bool(torch.isnan(got).all())             # nothing was launched
 
 
+def test_k_slices_summed_inside_the_kernel_equal_the_reduction_kernel(pkg):
+    """With the library's own scratch the slice of a tile that arrives last adds the slices up
+    inside the kernel; with a caller's workspace (whose arrival counters cannot be relied on) a
+    reduction kernel follows.  Both add in slice order: equal bit for bit, on ragged shapes, on
+    every tile shape the planner picks for them, and on every one of several launches in a row
+    (the counters are back at zero after each)."""
+    import torch
+    L = pkg.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    shapes = [(300, 4096, 500), (100, 8192, 1000), (257, 4096, 1023), (1000, 8192, 1000), (64, 28672, 8192),
+              (64, 8192, 10240), (256, 8192, 10240), (7168, 7168, 7168)]
+    for (M, K, N) in shapes:
+        assert pkg.plan(M, K, N)[0] == pkg.ALGO_TILE and pkg.plan(M, K, N)[2] > 1
+        need = L.fp8gemm_scratch_bytes(M, K, N)
+        dA = torch.from_numpy(pkg.fill((M, K), 0, seed=0xA11CE + 900 + M, dist="normal", sigma=2.0)).cuda()
+        dB = torch.from_numpy(pkg.fill((N, K), 1, seed=0xB0B + 900 + N, dist="normal", sigma=2.0)).cuda()
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        ref = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        assert L.fp8gemm_launch_ws(M, K, N, dA.data_ptr(), 0, dB.data_ptr(), 1, ref.data_ptr(), 2,
+                                   ws.data_ptr(), need, stream) == 0
+        outs = [torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda") for _ in range(4)]
+        for out in outs:
+            pkg.gemm(dA, dB, out=out, a_fmt=0, b_fmt=1)
+        torch.cuda.synchronize()
+        assert not bool(torch.isnan(ref).any())
+        for out in outs:
+            assert torch.equal(out, ref), (M, K, N)
+        del dA, dB, ws, ref, outs
+
+
 def test_back_to_back_launches_without_synchronisation(pkg, oracle):
     """Twenty launches of alternating shapes queued on one stream with no host
     synchronisation in between (stream order is the only ordering): each output is right."""
