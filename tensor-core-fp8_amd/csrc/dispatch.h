@@ -38,7 +38,6 @@ using TileQ4 = TileShape<128, 128, 64, 2, 2, 4, 2>;
 // and 6 slots run alike, 64-byte K tiles in an 8-deep ring 57 us, a 64 x 256 tile 54 us)
 using TileE5 = TileShape<64, 128, 128, 1, 4, 5, 3>;    // up to 64 rows of A: four waves of 64 x 32, 5 x 24 KiB ring
 using TileQ4s = TileShape<128, 128, 128, 2, 2, 4, 3>;  // up to 128 rows: the quarter tile with a 4 x 32 KiB ring
-using TileW6 = TileShape<256, 128, 64, 2, 2, 6, 2>;    // half-width tile, 6 x 24 KiB ring
 
 // Skinny kernel shapes: <MT, TN, BK, stages>.
 template <int MT, int TN>
@@ -229,7 +228,6 @@ hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, 
         return launch_ptile_shape<TileT2h, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
     case 15: return launch_ptile_shape<TileE5, AF, BF, false, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
     case 16: return launch_ptile_shape<TileQ4s, AF, BF, false, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
-    case 17: return launch_ptile_shape<TileW6, AF, BF, false, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
     default: return hipErrorInvalidValue;
     }
 }

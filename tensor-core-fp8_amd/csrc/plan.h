@@ -16,7 +16,7 @@ namespace fp8gemm_detail {
 
 // tiled kernel shapes: 0 P2, 1 P4, 2 P8, 3 S2, 4 S4, 5 H3, 6 Q2, 7 S64, 8 W3, 9 T2, 10 T4, 11 H4, 12 Q4, 13 P2h, 14 T2h,
 // 15 E5, 16 Q4s
-constexpr int kNumTileVariants = 18;
+constexpr int kNumTileVariants = 17;
 constexpr int kNumSkinnyVariants = 6;
 
 // Work list of the persistent kernel for a tile shape: `bulk` tiles (a multiple of 256)
