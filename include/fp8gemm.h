@@ -106,8 +106,11 @@ int fp8gemm_launch_ex(int m, int k, int n, const void *a, int a_fmt, const void 
  * (see fp8gemm_scratch_bytes) is refused with hipErrorOutOfMemory (2) before anything is
  * launched.  All calls on one GPU share that GPU's array: calls on one stream are ordered by
  * the stream, calls that overlap on different streams of one GPU race on it and must be
- * ordered by the caller.  Nothing in the array has to start at zero (every slot a call reads
- * has been written by that call), so none of it is ever cleared.
+ * ordered by the caller.  The first 16 KiB of the array are the arrival counters of the K
+ * slices: they must be zero when a kernel starts, they are (static storage starts as zeros),
+ * and the slice that arrives last puts its tile's counter back to zero, so every kernel
+ * leaves them as it found them; nothing else in the array has to start at any value
+ * (every slot a call reads has been written by that call).
  */
 #define FP8GEMM_NOALLOC_SCRATCH_BYTES ((size_t)64 << 20)
 int fp8gemm_launch_noalloc(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
@@ -163,10 +166,15 @@ int fp8gemm_tile_order(int m, int k, int n, int bm, int bn, int index, int *tile
 
 /*
  * Device scratch.  A shape whose plan cuts K into slices needs device memory for the
- * slices' partial sums between its two kernels; fp8gemm_scratch_bytes tells how much
- * (0 when the shape needs none: 8192^3, M=16 N=28672 K=8192, ...; the figure is for the
- * stage-2 plan, the stage-4 plan cuts K the same way).  It is the only device memory the
- * library ever allocates.  The reference's launchers are stateless and re-entrant
+ * slices' partial sums; fp8gemm_scratch_bytes tells how much (0 when the shape needs
+ * none: 8192^3, M=16 N=28672 K=8192, ...; the figure is for the stage-2 plan, the stage-4
+ * plan cuts K the same way; it includes 16 KiB of arrival counters ahead of the sums).
+ * With the library's own scratch the slices of tiles up to 128 x 128 are added up inside the
+ * GEMM kernel, by the slice of a tile that arrives last (the counters start at zero and
+ * every kernel leaves them at zero); larger tiles, and every shape run on a caller's
+ * workspace, whose contents the library cannot vouch for, are added up by a second kernel.
+ * Both add in slice order: the results are the same bit for bit.  The scratch is the only
+ * device memory the library ever allocates.  The reference's launchers are stateless and re-entrant
  * (GEMM/src/gemm.cu:263-277); to keep that contract the scratch is held per (device,
  * stream): calls on one stream are ordered by the stream, calls on different streams
  * never share a buffer and may overlap freely, from one host thread or several.  A

@@ -18,6 +18,7 @@ import subprocess
 E4M3 = 0
 E5M2 = 1
 ALGO_AUTO, ALGO_DIRECT, ALGO_TILE, ALGO_SKINNY = 0, 1, 2, 3
+NOALLOC_SCRATCH_BYTES = 64 << 20      # FP8GEMM_NOALLOC_SCRATCH_BYTES: the static array behind fp8gemm_launch_noalloc
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libfp8gemm.so")

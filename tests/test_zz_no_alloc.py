@@ -66,3 +66,53 @@ def test_noalloc_entry_refuses_what_the_static_array_cannot_hold(pkg):
     assert bool(torch.isnan(out).all())
     assert noalloc(0, K, N, dA.data_ptr(), 0, dB.data_ptr(), 0, out.data_ptr(), 2, stream) == 1
     assert noalloc(M, K, N, None, 0, dB.data_ptr(), 0, out.data_ptr(), 2, stream) == 1
+
+
+def test_noalloc_entry_under_graph_capture_and_replay(pkg):
+    """What the entry point is for: K-sliced launches captured into a HIP graph (tiles whose
+    slices are added up inside the kernel, and tiles that take the reduction kernel), replayed
+    several times with eager launches of other shapes and synchronisations in between.  Every
+    replay must reproduce the eager result bit for bit: the arrival counters are back at zero
+    after each launch, nothing is cleared from the host, nothing is allocated."""
+    import torch
+    L = pkg.lib()
+    noalloc = _bind(L)
+    shapes = [(64, 8192, 2048), (256, 8192, 2048), (100, 8192, 1000), (16, 4096, 512)]
+    side = torch.cuda.Stream()
+    cases = []
+    for (M, K, N) in shapes:
+        dA = torch.from_numpy(pkg.fill((M, K), 0, seed=0xA11CE + 800 + N, dist="normal", sigma=2.0)).cuda()
+        dB = torch.from_numpy(pkg.fill((N, K), 1, seed=0xB0B + 800 + N, dist="normal", sigma=2.0)).cuda()
+        ref = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        pkg.gemm(dA, dB, out=ref, a_fmt=0, b_fmt=1)
+        got = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        cases.append((M, K, N, dA, dB, ref, got))
+    assert any(pkg.plan(M, K, N)[2] > 1 for (M, K, N) in shapes)
+    torch.cuda.synchronize()
+
+    def enqueue():
+        for (M, K, N, dA, dB, ref, got) in cases:
+            assert noalloc(M, K, N, dA.data_ptr(), 0, dB.data_ptr(), 1, got.data_ptr(), 2, side.cuda_stream) == 0
+    with torch.cuda.stream(side):
+        enqueue()                  # eager, before the capture: the static array's address is looked up here
+    side.synchronize()
+    for (M, K, N, dA, dB, ref, got) in cases:
+        assert torch.equal(got, ref), ("eager", M, K, N)
+    held = L.fp8gemm_scratch_held_bytes()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        enqueue()
+    other = cases[1]
+    for replay in range(4):
+        for (M, K, N, dA, dB, ref, got) in cases:
+            got.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        for (M, K, N, dA, dB, ref, got) in cases:
+            assert torch.equal(got, ref), (replay, M, K, N)
+        # eager work of the program's own between the replays, on the default stream
+        tmp = torch.empty_like(other[5])
+        pkg.gemm(other[3], other[4], out=tmp, a_fmt=0, b_fmt=1)
+        torch.cuda.synchronize()
+        assert torch.equal(tmp, other[5])
+    assert L.fp8gemm_scratch_held_bytes() == held
