@@ -216,17 +216,53 @@ SkinnyPlan plan_skinny(int m, int k, int n)
         while ((long)(n / (16 * tn)) * split < 448 && split < 16 && ksteps % (2 * split) == 0 && ksteps / (2 * split) >= 32)
             split *= 2;
     } else {
-        while (tn > 1 && (n % (16 * tn) != 0 || n / (16 * tn) < 256)) tn /= 2;
-        while (n % (16 * tn) != 0) tn /= 2;
-        while ((long)(n / (16 * tn)) * split < 192 && split < 16 && ksteps % (2 * split) == 0 && ksteps / (2 * split) >= 8)
+        // Streams of 64, 32 or 16 columns: the widest that still gives 400 streams or more (every
+        // stream re-reads A, and a wide stream's ring holds more of B per load instruction); with
+        // more than a few rows of A, a count that fills the 256 CUs evenly (a multiple of 256) is
+        // taken before that; failing both, the count that loads the CUs most evenly, the wider
+        // streams on a tie.  Measured (cold, us) for 64 / 32 / 16 columns: M=1 N=10240 K=8192
+        // 16.9 / 17.6 / 15.6, M=16 18.4 / 19.4 / 17.5; M=1 N=8192 K=28672 37.4 / 37.5 / 35.6,
+        // M=16 38.8 / 37.5 / 38.1; M=16 N=6144 K=8192 - / 11.3 / 12.6; N=28672 is best at 64.
+        int pick = 0;
+        for (int t = 4; t >= 1 && !pick; t /= 2) {
+            if (n % (16 * t) != 0) continue;
+            const int streams = n / (16 * t);
+            if (streams >= 400 || (m > 4 && streams >= 256 && streams % 256 == 0)) pick = t;
+        }
+        if (!pick) {
+            double best = -1.0;
+            for (int t = 4; t >= 1; t /= 2) {
+                if (n % (16 * t) != 0) continue;
+                const int streams = n / (16 * t);
+                const double even = (double)streams / (256.0 * ((streams + 255) / 256));
+                if (even > best + 1e-9) {
+                    best = even;
+                    pick = t;
+                }
+            }
+        }
+        tn = pick;
+        // (K slices cost a second launch, about 2.5 us: only while there are fewer streams than CUs
+        // and a slice keeps 4 KiB of K or more)
+        while ((long)(n / (16 * tn)) * split < 256 && split < 16 && ksteps % (2 * split) == 0 && ksteps / (2 * split) >= 32)
             split *= 2;
     }
     p.tn = tn;
     p.nsplit = split;
     const int kchunk = k / split;
-    // fat streams (64 columns) run best on 128-byte K steps in a deep ring; thinner ones want
-    // longer K steps, so that a ring stage still holds 16 KiB or more
-    p.variant = (tn == 4 && p.mt <= 3) ? 0 : (kchunk % 512 == 0) ? 4 : (kchunk % 256 == 0) ? 1 : 0;
+    const long waves = (long)(n / (16 * tn)) * split;
+    // Fat streams (64 columns) run best on 128-byte K steps in a deep ring; thinner ones want
+    // longer K steps, so that a ring stage still holds 16 KiB or more: the thinnest, on a long K
+    // and with two waves or more per CU, whole 1 KiB rows.  Three waves or more per CU on a
+    // short K: a ring small enough for all of them to be resident at once.
+    if (tn == 4 && p.mt <= 3)
+        p.variant = 0;
+    else if (tn == 1 && kchunk % 1024 == 0 && kchunk >= 8192 && waves >= 512)
+        p.variant = 5;
+    else if (waves > 512 && kchunk < 8192)
+        p.variant = kchunk % 256 == 0 ? 1 : 0;
+    else
+        p.variant = (kchunk % 512 == 0) ? 4 : (kchunk % 256 == 0) ? 1 : 0;
     return p;
 }
 
