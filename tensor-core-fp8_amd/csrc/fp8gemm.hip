@@ -38,15 +38,28 @@ constexpr int kPlannedCus = 256;
 constexpr int kMaxDevices = 64;
 
 // ------------------------------------------------------------------ scratch
+__global__ void zero_ints_kernel(int *p, int count)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) p[i] = 0;
+}
+
 // Device runtime behind the scratch bookkeeping (scratch_pool.h).
 struct HipScratchBackend {
     using Event = hipEvent_t;
-    // (a new buffer starts with zeroed arrival counters; the kernels leave them at zero)
-    int alloc(size_t bytes, void **ptr)
+    // A new buffer starts with zeroed arrival counters (the kernels leave them at zero).  They
+    // are cleared by a kernel on the stream that asked for the buffer: ordered before that
+    // stream's GEMM, without the host or any other stream waiting (a hipMemset would run on the
+    // null stream, which a non-blocking stream is not ordered against).
+    int alloc(size_t bytes, void *stream, void **ptr)
     {
         hipError_t e = hipMalloc(ptr, bytes);
         if (e != hipSuccess) return (int)e;
-        e = hipMemset(*ptr, 0, bytes < kSliceCounterBytes ? bytes : kSliceCounterBytes);
+        const size_t ints = (bytes < kSliceCounterBytes ? bytes : kSliceCounterBytes) / sizeof(int);
+        (void)hipGetLastError();
+        hipLaunchKernelGGL(zero_ints_kernel, dim3((unsigned)((ints + 255) / 256)), dim3(256), 0,
+                           static_cast<hipStream_t>(stream), static_cast<int *>(*ptr), (int)ints);
+        e = hipGetLastError();
         if (e != hipSuccess) (void)hipFree(*ptr);
         return (int)e;
     }

@@ -17,7 +17,8 @@
 //
 // The device runtime is reached through a Backend type, so the bookkeeping can be
 // exercised on the host with a fake one:
-//   int  alloc(size_t bytes, void **ptr)        0 on success, else an error code
+//   int  alloc(size_t bytes, void *stream, void **ptr)   a new buffer, made ready for use by work queued on
+//                                               `stream` from now on; 0 on success, else an error code
 //   void free(void *ptr)
 //   int  record(void *stream, Event *ev)        marks what `stream` has queued so far
 //   bool passed(Event ev)                       true once that work is done
@@ -78,7 +79,7 @@ public:
             const size_t granule = (size_t)2 << 20;
             const size_t want = (bytes + granule - 1) / granule * granule;
             void *p = nullptr;
-            const int e = backend_.alloc(want, &p);
+            const int e = backend_.alloc(want, stream, &p);
             if (e != 0) return e;
             slot->ptr = p;
             slot->bytes = want;

@@ -30,7 +30,7 @@ struct FakeState {
 struct FakeBackend {
     using Event = int;
     FakeState *st;
-    int alloc(size_t bytes, void **ptr)
+    int alloc(size_t bytes, void *, void **ptr)
     {
         if (st->fail_alloc) return 2;
         *ptr = std::malloc(16);
