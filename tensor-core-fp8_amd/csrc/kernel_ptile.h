@@ -177,7 +177,8 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
     // K slices each (slice-major item order: neighbours are still neighbouring tiles);
     // every round of such items is spread evenly over the eight XCDs.  Slice s of tail
     // tile u writes its partial sums to slot s*tail + u of the scratch `ws` (BM x BN
-    // floats, row stride BN; the host adds the slices up afterwards); unsplit items
+    // floats, row stride BN; the slices are added up by the one that arrives last, see the end of
+    // the item, or by a reduction kernel that the host launches afterwards); unsplit items
     // write C directly.
     const int xcd = blockIdx.x & 7;
     const int slot = blockIdx.x >> 3;
