@@ -222,10 +222,10 @@ hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, 
     case 12: return launch_ptile_shape<TileQ4, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
     case 13:
         if (!p2h_ok(k, nsplit)) return hipErrorInvalidValue;
-        return launch_ptile_shape<TileP2h, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+        return launch_ptile_shape<TileP2h, AF, BF, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
     case 14:
         if (!p2h_ok(k, nsplit)) return hipErrorInvalidValue;
-        return launch_ptile_shape<TileT2h, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
+        return launch_ptile_shape<TileT2h, AF, BF, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
     case 15: return launch_ptile_shape<TileE5, AF, BF, false, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
     case 16: return launch_ptile_shape<TileQ4s, AF, BF, false, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
     default: return hipErrorInvalidValue;

@@ -200,7 +200,7 @@ bool plain_output(const OutSpec &spec)
 
 bool p2h_ok(int k, int nsplit)
 {
-    return k % 128 == 0 && (k / 128) / nsplit >= 2;
+    return k % 16 == 0 && ((k + 127) / 128) / nsplit >= 2;
 }
 
 // the single-wave streams, up to 64 rows
@@ -341,9 +341,10 @@ TilePlan plan_tile(int m, int k, int n, int stages)
         if (m <= 64 && k % 128 == 0 && c.variant != 15) continue;
         if (stages == 4) {
             // the 4-deep rings rank like their 2- and 3-deep twins (same tiles, same work list);
-            // only the 256 x 256 one is compiled for a K that is not a multiple of its K tile
-            if (c.variant4 < 0 || (k % 64 != 0 && c.variant4 != 1)) continue;
-        } else if (k % 128 != 0 && !(c.variant == 0 || c.variant == 5 || c.variant == 6)) {
+            // only the 256 x 256 one (and the 16x16x128 kernels they share with the 2-stage entry
+            // points) is compiled for a K that is not a multiple of its K tile
+            if (c.variant4 < 0 || (k % 64 != 0 && !(c.variant4 == 1 || c.variant4 == 13 || c.variant4 == 14))) continue;
+        } else if (k % 128 != 0 && !(c.variant == 0 || c.variant == 5 || c.variant == 6 || c.variant == 13 || c.variant == 14)) {
             continue;      // overhanging K tile: only the shapes compiled for it
         }
         for (int mode = 0; mode < 2; ++mode)          // 0: slices for the tail tiles only, 1: for all

@@ -37,8 +37,8 @@ size_t ptile_scratch_bytes(const PtileWork &w, int bm, int bn);
 
 // the plain entry points: bare fp32 sums, no scaling
 bool plain_output(const OutSpec &spec);
-// The 16x16x128 forms of the 256 x 256 and 192 x 256 tiles need whole 128-byte K tiles, at least two per
-// work item (a tile, or one of its nsplit K slices).
+// The 16x16x128 forms of the 256 x 256 and 192 x 256 tiles need at least two 128-byte K tiles per work
+// item (a tile, or one of its nsplit K slices); the last K tile may overhang a K that is a multiple of 16.
 bool p2h_ok(int k, int nsplit);
 
 struct SkinnyPlan {

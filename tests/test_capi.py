@@ -71,9 +71,9 @@ def test_kernel_selection_is_pure_host_logic(pkg):
     assert s == 0 or (s - COUNTERS) % (16 * 8192 * 4) == 0        # whole partial-sum planes, or none
     # the plan behind the automatic selection: family, variant, K slices, columns | rotation
     assert pkg.plan(8192, 8192, 8192) == (pkg.ALGO_TILE, 13, 1, 2)         # 256x256 persistent tiles on the 16x16x128 MFMA, no slices
-    assert pkg.plan(8192, 8256, 8192) == (pkg.ALGO_TILE, 0, 1, 2)          # K not a multiple of 128: the 32x32x64 form
+    assert pkg.plan(8192, 8256, 8192) == (pkg.ALGO_TILE, 13, 1, 2)         # K not a multiple of 128: the same kernel, the last K tile overhangs
     assert pkg.plan(8192, 8192, 8192, stages=4)[:3] == (pkg.ALGO_TILE, 13, 1)        # shared with the 2-stage entry points
-    assert pkg.plan(8192, 8256, 8192, stages=4)[:3] == (pkg.ALGO_TILE, 1, 1)         # 4-deep ring of 64-byte K tiles
+    assert pkg.plan(8192, 8256, 8192, stages=4)[:3] == (pkg.ALGO_TILE, 13, 1)        # ... for both entry points
     fam, var, slices, cols = pkg.plan(16, 8192, 28672)
     assert (fam, slices, cols) == (pkg.ALGO_SKINNY, 1, 64)
     fam, var, slices, _ = pkg.plan(256, 28672, 8192)

@@ -151,6 +151,25 @@ def test_tile_variant_on_16x16x128_mfma(pkg, oracle, variant, fa, fb, shape):
     assert_within_bound(oracle, C, A, fa, B, fb, hw_term=True)
 
 
+@pytest.mark.parametrize("fa,fb", PAIRS)
+@pytest.mark.parametrize("variant", [13, 14])
+@pytest.mark.parametrize("shape", [(300, 144, 200), (512, 2000, 520), (1100, 4112, 700), (256, 8256, 512), (700, 1216, 300)])
+def test_16x16x128_variants_with_an_overhanging_last_k_tile(pkg, oracle, variant, fa, fb, shape):
+    """K a multiple of 16 but not of 128 (even and odd counts of K tiles, K a multiple of 64 or
+    not): the bytes of the last K tile past the end of each row count as zeros in the
+    16x16x128 kernels as well, all four pairings; K slices over such a K included."""
+    M, K, N = shape
+    assert K % 16 == 0 and K % 128 != 0
+    A = pkg.fill((M, K), fa, seed=0xA11CE + K + variant, dist="normal", sigma=4.0)
+    B = pkg.fill((N, K), fb, seed=0xB0B + K + variant, dist="normal", sigma=4.0)
+    C = run_gpu(pkg, A, fa, B, fb, algo=ALGOS["tile"], variant=variant)
+    worst = assert_within_bound(oracle, C, A, fa, B, fb, hw_term=K < 1024)
+    assert worst < 0.5
+    if (K + 127) // 128 >= 4:
+        C2 = run_gpu(pkg, A, fa, B, fb, algo=ALGOS["tile"], variant=variant, split_k=2)
+        assert_within_bound(oracle, C2, A, fa, B, fb, hw_term=K < 1024)
+
+
 @pytest.mark.parametrize("variant", [13, 14])
 def test_16x16x128_variant_refuses_a_single_k_tile(pkg, variant):
     A = np.zeros((256, 128), np.uint8)
