@@ -67,6 +67,15 @@ int fp8gemm_launch(int m, int k, int n, const void *a, int a_fmt, const void *b,
                    float *out, int stages, void *stream);
 
 /*
+ * Matrix-vector product y = W x: W stored n x k row-major (the layout of B above), x of k
+ * codes, y of n floats.  The GEMV that the reference's roadmap names next to GEMM
+ * (README.md:7 there; it holds no GEMV code to match).  It is fp8gemm_launch with m = 1:
+ * the single-wave streaming kernel reads every byte of W once (k % 128 == 0 and n % 16 == 0;
+ * any other shape runs on the tiled or the general kernel).
+ */
+int fp8gemm_gemv(int n, int k, const void *w, int w_fmt, const void *x, int x_fmt, float *y, void *stream);
+
+/*
  * Extended epilogue, with no counterpart in the reference's gemm:: API; it covers what the
  * reference's vendor-library sample hands to cuBLASLt next to the operands
  * (GEMM/src/cublas.cu:9-23, 41-46; GEMM/include/helper.h:84, 125, 159-160: host alpha and

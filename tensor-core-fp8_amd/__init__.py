@@ -67,6 +67,8 @@ def lib():
         fn.argtypes = [ci, ci, ci, vp, vp, vp]
     L.fp8gemm_launch.restype = ci
     L.fp8gemm_launch.argtypes = [ci, ci, ci, vp, ci, vp, ci, vp, ci, vp]
+    L.fp8gemm_gemv.restype = ci
+    L.fp8gemm_gemv.argtypes = [ci, ci, vp, ci, vp, ci, vp, vp]
     L.fp8gemm_launch_ws.restype = ci
     L.fp8gemm_launch_ws.argtypes = [ci, ci, ci, vp, ci, vp, ci, vp, ci, vp, ctypes.c_size_t, vp]
     L.fp8gemm_launch_noalloc.restype = ci

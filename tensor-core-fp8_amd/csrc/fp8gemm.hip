@@ -447,6 +447,11 @@ int fp8gemm_launch(int m, int k, int n, const void *a, int a_fmt, const void *b,
     return launch_pooled(m, k, n, a, a_fmt, b, b_fmt, out, stages, FP8GEMM_ALGO_AUTO, -1, 0, stream);
 }
 
+int fp8gemm_gemv(int n, int k, const void *w, int w_fmt, const void *x, int x_fmt, float *y, void *stream)
+{
+    return launch_pooled(1, k, n, x, x_fmt, w, w_fmt, y, 2, FP8GEMM_ALGO_AUTO, -1, 0, stream);
+}
+
 int fp8gemm_launch_ws(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
                       float *out, int stages, void *workspace, size_t workspace_bytes, void *stream)
 {

@@ -530,6 +530,30 @@ def test_k_slices_summed_inside_the_kernel_equal_the_reduction_kernel(pkg):
         del dA, dB, ws, ref, outs
 
 
+@pytest.mark.parametrize("fw,fx", PAIRS)
+@pytest.mark.parametrize("shape", [(4096, 4096), (10240, 8192), (1000, 8192), (512, 1040), (333, 777), (28672, 2048)])
+def test_gemv_entry_point(pkg, oracle, fw, fx, shape):
+    """fp8gemm_gemv: y = W x against the CPU loop with one row of A (all four pairings; shapes
+    the streaming kernel takes, shapes that fall to the tiled kernel and to the general one),
+    and bit-equal to fp8gemm_launch with m = 1."""
+    import torch
+    L = pkg.lib()
+    N, K = shape
+    W = pkg.fill((N, K), fw, seed=0xB0B + 1100 + N, dist="normal", sigma=2.0)
+    x = pkg.fill((1, K), fx, seed=0xA11CE + 1100 + K, dist="normal", sigma=2.0)
+    dW, dx = torch.from_numpy(W).cuda(), torch.from_numpy(x).cuda()
+    y = torch.full((N,), float("nan"), dtype=torch.float32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    assert L.fp8gemm_gemv(N, K, dW.data_ptr(), fw, dx.data_ptr(), fx, y.data_ptr(), stream) == 0
+    ref = torch.full((1, N), float("nan"), dtype=torch.float32, device="cuda")
+    assert L.fp8gemm_launch(1, K, N, dx.data_ptr(), fx, dW.data_ptr(), fw, ref.data_ptr(), 2, stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(y, ref[0])
+    assert_within_bound(oracle, y.cpu().numpy()[None, :], x, fx, W, fw, hw_term=K < 1024)
+    assert L.fp8gemm_gemv(0, K, dW.data_ptr(), fw, dx.data_ptr(), fx, y.data_ptr(), stream) == 1
+    assert L.fp8gemm_gemv(N, K, None, fw, dx.data_ptr(), fx, y.data_ptr(), stream) == 1
+
+
 def test_back_to_back_launches_without_synchronisation(pkg, oracle):
     """Twenty launches of alternating shapes queued on one stream with no host
     synchronisation in between (stream order is the only ordering): each output is right."""
