@@ -37,8 +37,8 @@ SHAPES = [
     (256, 1024, 512),       # persistent tiled kernel, whole tiles
     (300, 2048, 250),       # tiles that overhang C (n not a multiple of 4: guarded element stores)
     (16, 4096, 1024),       # weight-streaming kernel
-    (48, 8192, 256),        # weight-streaming kernel with K slices + reduction
-    (256, 8192, 1024),      # tiled kernel with K slices + tile-slot reduction
+    (48, 8192, 256),        # 64 x 128 weight-streaming tiles with K slices, summed inside the kernel
+    (256, 8192, 1024),      # 128 x 128 tiles with K slices, summed inside the kernel
     (70, 200, 90),          # general kernel (k not a multiple of 16)
     (512, 1040, 384),       # K tile overhanging K
     (3584, 256, 3584),      # 256 x 256 tiles on the 16x16x128 MFMA
@@ -121,20 +121,18 @@ EPI_SHAPES = [
     (256, 1024, 512),       # persistent tiled kernel, whole tiles
     (300, 2048, 250),       # tiles that overhang C, n not a multiple of 4
     (16, 4096, 1024),       # weight-streaming kernel
-    (48, 8192, 256),        # weight-streaming kernel with K slices + reduction
-    (256, 8192, 1024),      # tiled kernel with K slices + tile-slot reduction
+    (48, 8192, 256),        # 64 x 128 weight-streaming tiles with K slices, summed inside the kernel
+    (256, 8192, 1024),      # 128 x 128 tiles with K slices, summed inside the kernel
     (70, 200, 90),          # general kernel
     (3584, 256, 3584),      # 256 x 256 tiles on the 16x16x128 MFMA
 ]
 
 
-@pytest.mark.parametrize("d_dtype,c_dtype", [("float32", "float32"), ("bfloat16", "float32"), ("float16", "bfloat16"),
-                                             ("float32", "float16")])
-@pytest.mark.parametrize("shape", EPI_SHAPES)
-def test_beta_c_d_scale_and_amax(pkg, oracle, shape, d_dtype, c_dtype):
+def check_full_epilogue(pkg, oracle, shape, d_dtype, c_dtype, rows=None):
     """d = cast(sd * (alpha*sa*sb*sum + beta*sc*C)), amax = max|.| before sd: against the oracle's
     sum within the fp32 reordering bound carried through the epilogue, plus the rounding of the
-    epilogue's own fp32 operations and half an ulp of the output format."""
+    epilogue's own fp32 operations and half an ulp of the output format.  rows: check these rows
+    of the result only (amax is then bounded from below by them)."""
     M, K, N = shape
     fa, fb = (0, 1) if K % 3 else (1, 0)
     A = pkg.fill((M, K), fa, seed=0xA11CE + 600 + K, dist="normal", sigma=1.0)
@@ -143,7 +141,12 @@ def test_beta_c_d_scale_and_amax(pkg, oracle, shape, d_dtype, c_dtype):
     Cin = (rng.standard_normal((M, N)) * 40.0).astype(np.float32)
     alpha, beta, sa, sb, sc, sd = 0.5, -1.5, 0.125, 3.0, 0.75, 0.0625
     got, amax, c_used = run_full(pkg, A, fa, B, fb, d_dtype, alpha, beta, Cin, c_dtype, sa, sb, sc, sd)
-    Cref, S = oracle.gemm(A, fa, B, fb, with_scale=True)
+    assert np.isfinite(got).all()
+    if rows is None:
+        Cref, S = oracle.gemm(A, fa, B, fb, with_scale=True)
+    else:
+        Cref, S = oracle.gemm(A, fa, B, fb, rows=rows, with_scale=True)
+        got, c_used = got[rows], c_used[rows]
     fab = float(np.float32(np.float32(alpha) * np.float32(sa)) * np.float32(sb))
     fc = float(np.float32(beta) * np.float32(sc))
     y = fab * Cref.astype(np.float64) + fc * c_used
@@ -152,12 +155,31 @@ def test_beta_c_d_scale_and_amax(pkg, oracle, shape, d_dtype, c_dtype):
     want = sd * y
     mant, emin = FORMATS[d_dtype]
     bound = sd * ytol + 0.5 * ulp16(np.abs(want) + sd * ytol, mant, emin) + np.abs(want) * 2.0 ** -23
-    assert np.isfinite(got).all()
     err = np.abs(got - want)
     assert (err <= bound).all(), "worst err/bound = %g" % float((err / bound).max())
     # amax: the largest |y| (before sd), within the tolerance of the element that attains it
     assert amax is not None and amax > 0
-    assert abs(amax - np.abs(y).max()) <= ytol.max() + np.abs(y).max() * 2.0 ** -22
+    if rows is None:
+        assert abs(amax - np.abs(y).max()) <= ytol.max() + np.abs(y).max() * 2.0 ** -22
+    else:
+        assert amax >= np.abs(y).max() - ytol.max() - np.abs(y).max() * 2.0 ** -22
+
+
+@pytest.mark.parametrize("d_dtype,c_dtype", [("float32", "float32"), ("bfloat16", "float32"), ("float16", "bfloat16"),
+                                             ("float32", "float16")])
+@pytest.mark.parametrize("shape", EPI_SHAPES)
+def test_beta_c_d_scale_and_amax(pkg, oracle, shape, d_dtype, c_dtype):
+    check_full_epilogue(pkg, oracle, shape, d_dtype, c_dtype)
+
+
+@pytest.mark.parametrize("d_dtype,c_dtype", [("bfloat16", "float32"), ("float32", "float16")])
+def test_epilogue_in_the_reduction_kernel(pkg, oracle, d_dtype, c_dtype):
+    """128 x 256 tiles in 8 K slices: too large for the in-kernel sum, so the slices are added up,
+    and the epilogue applied, by the reduction kernel (sampled rows against the oracle)."""
+    shape = (256, 16384, 4096)
+    fam, var, slices, _ = pkg.plan(*shape)
+    assert fam == pkg.ALGO_TILE and var in (5, 8, 0, 13) and slices > 1
+    check_full_epilogue(pkg, oracle, shape, d_dtype, c_dtype, rows=np.arange(0, 256, 8, dtype=np.int32))
 
 
 @pytest.mark.parametrize("shape", [(256, 512, 256), (16, 1024, 512), (100, 256, 60), (48, 8192, 256), (256, 8192, 1024)])
