@@ -223,10 +223,29 @@ bool run_size(hipblasLtHandle_t handle, Problem &p, int repeat, bool comparable)
 int main(int argc, char *argv[])
 {
     if (argc < 2) {
-        printf("Usage: %s <repeat> [first last step] [sample]\n", argv[0]);
+        printf("Usage: %s <repeat> [first last step] [sample]\n       %s <repeat> shape M K N\n", argv[0], argv[0]);
         return 1;
     }
     const int repeat = atoi(argv[1]);
+    if (argc == 6 && strcmp(argv[2], "shape") == 0) {
+        // one shape that need not be square (same weight buffer for every launch)
+        const int m = atoi(argv[3]), k = atoi(argv[4]), n = atoi(argv[5]);
+        if (repeat < 1 || m < 1 || k < 1 || n < 1) {
+            printf("bad arguments\n");
+            return 1;
+        }
+        try {
+            hipblasLtHandle_t handle = nullptr;
+            check_lt(hipblasLtCreate(&handle), "create");
+            Problem p(m, n, k, 1.0f, 0.0f, 1.0f, 1.0f, 32ull * 1024 * 1024);
+            run_size(handle, p, repeat, true);
+            check_lt(hipblasLtDestroy(handle), "destroy");
+        } catch (const std::exception &e) {
+            printf("aborted: %s\n", e.what());
+            return 2;
+        }
+        return 0;
+    }
     int first = 256, last = 16384, step = 256;
     bool sample = false;
     int pos = 2;
