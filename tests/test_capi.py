@@ -171,3 +171,43 @@ def test_tile_order_is_a_bijection_with_compact_windows(pkg):
         L.fp8gemm_tile_order(4352, 12288, 16384, 256, 256, g, ctypes.byref(tr), ctypes.byref(tc))
         first[g] = (tr.value, tc.value)
     assert {r for r, _ in first} == set(range(16)) and {c for _, c in first} == set(range(16))
+
+
+def test_plans_are_consistent_over_random_shapes(pkg):
+    """Host-only sweep of the planner: whatever it picks can run the shape.  Streams: m <= 16,
+    a column count per wave of 16, 32 or 64 that divides n, K slices that are whole 128-byte K
+    steps.  Tiles: a compiled variant, slices only where K has K tiles to spare, scratch within
+    the cap.  The scratch query agrees with the plan (arrival counters + whole fp32 planes / slots)."""
+    L = pkg.lib()
+    rng = np.random.default_rng(20240611)
+    COUNTERS = 16 * 1024
+    n_tile_variants = L.fp8gemm_num_variants(pkg.ALGO_TILE)
+    n_stream_variants = L.fp8gemm_num_variants(pkg.ALGO_SKINNY)
+    shapes = [(1, 8192, 10240), (16, 28672, 1024), (4, 16384, 2048), (16, 14336, 512), (17, 128, 16), (16, 128, 16)]
+    for _ in range(3000):
+        m = int(rng.choice([1, 2, 7, 16, 17, 33, 64, 100, 128, 256, 300, 1000, 4096, 5000]))
+        k = int(rng.integers(1, 260)) * int(rng.choice([16, 64, 128]))
+        n = int(rng.integers(1, 1800)) * int(rng.choice([1, 16, 16, 128]))
+        shapes.append((m, k, n))
+    for (m, k, n) in shapes:
+        for stages in (2, 4):
+            fam, var, slices, extra = pkg.plan(m, k, n, stages)
+            assert fam == L.fp8gemm_select_algo(m, k, n)
+            assert slices >= 1
+            if fam == pkg.ALGO_SKINNY:
+                assert m <= 16 and k % 128 == 0 and n % 16 == 0
+                assert extra in (16, 32, 64) and n % extra == 0
+                assert 0 <= var < n_stream_variants
+                assert k % (128 * slices) == 0
+                if stages == 2:
+                    want = COUNTERS + slices * m * n * 4 if slices > 1 else 0
+                    assert L.fp8gemm_scratch_bytes(m, k, n) == want
+            elif fam == pkg.ALGO_TILE:
+                assert k % 16 == 0 and 0 <= var < n_tile_variants
+                assert slices == 1 or (k + 127) // 128 >= 2 * slices
+                if stages == 2:
+                    need = L.fp8gemm_scratch_bytes(m, k, n)
+                    assert (need > 0) == (slices > 1) and need <= (1 << 30) + COUNTERS
+                    assert need == 0 or (need - COUNTERS) % 4096 == 0
+            else:
+                assert fam == pkg.ALGO_DIRECT and slices == 1 and L.fp8gemm_scratch_bytes(m, k, n) == 0
