@@ -244,6 +244,22 @@ def main():
                   "pass": bool((err <= tol).all())}
     except Exception as ex:  # the oracle is only the checker; say so if it is unavailable
         parity = {"error": str(ex)[:200]}
+
+    # The same launch on all-zero operands: same instructions, same memory traffic, far less
+    # switching in the matrix pipe.  What it gains over the figure above is what the board's power
+    # limit takes from the kernel on real data (reported beside `value`, never as it).
+    A.zero_()
+    B.zero_()
+    zero_sampler = BoardSampler()
+    zero_sampler.start()
+    settle(torch, go)
+    zero_ms, _ = time_launches(torch, go, args.steps, args.warmup)
+    zero_sampler.stop_flag.set()
+    zero_sampler.join()
+    zero_operands = {"what": "the same kernel and shape on all-zero operands (not a result: it shows how much of the "
+                             "gap to the peak is the board's power limit on N(0,1) data)",
+                     "tflops": to_tflops(zero_ms), "frac_of_fp8_peak": to_tflops(zero_ms) / PEAK_FP8_TFLOPS,
+                     "board": zero_sampler.summary()}
     del A, B, C
 
     # ---------------------------------------------------------------- LLM-linear shapes, HBM-bound
@@ -413,6 +429,7 @@ def main():
         "repeats": {"what": "five more blocks of `steps` launches right after the timed one",
                     "tflops_median": rep_tf[2], "tflops_min": rep_tf[0], "tflops_max": rep_tf[-1]},
         "board": sampler.summary(),
+        "zero_operands": zero_operands,
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / PEAK_FP8_TFLOPS, "traffic": TRAFFIC_BYTES_8192,
                      "traffic_source": "constant from the rocprofv3 --pmc summary under profiles/ "
