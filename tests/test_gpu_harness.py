@@ -108,3 +108,32 @@ def test_make_gemm_test_target(pkg):
     r = subprocess.run(["make", "-C", pkg.HARNESS_DIR, "gemm_test"], capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stdout[-1500:] + r.stderr[-1500:]
     assert "Result Verified!" in r.stdout
+
+
+def test_vendor_comparator_runs_both_libraries_and_compares_them(pkg, tmp_path):
+    """`out/hipblaslt` (the counterpart of the reference's `out/cublas`, GEMM/src/cublas.cu with
+    GEMM/include/helper.h): hipBLASLt and this library on the same operands, both timed, the two
+    results compared.  Sweep mode on two small sizes, the single-shape mode on a skinny shape."""
+    exe = os.path.join(pkg.HARNESS_DIR, "out", "hipblaslt")
+    if not os.path.exists(exe):
+        raise RuntimeError("the comparator is not built (%s): run __graft_entry__.build()" % exe)
+
+    def run(*args):
+        r = subprocess.run([exe] + [str(a) for a in args], capture_output=True, text=True, cwd=str(tmp_path), timeout=300)
+        assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+        return r.stdout
+
+    def check(out, shapes):
+        vendor = re.findall(r"GEMM-hipblaslt-fp8: M\[(\d+)\] x N\[(\d+)\] x K\[(\d+)\], performance = ([0-9.]+)GFLOPS", out)
+        ours = re.findall(r"GEMM-fp8gemm-fp8:\s+M\[(\d+)\] x N\[(\d+)\] x K\[(\d+)\], performance = ([0-9.]+)GFLOPS", out)
+        diffs = re.findall(r"max \|hipblaslt - fp8gemm\| = ([0-9.eE+-]+) \(largest \|C\| = ([0-9.eE+-]+)", out)
+        assert [tuple(int(x) for x in v[:3]) for v in vendor] == shapes == [tuple(int(x) for x in v[:3]) for v in ours]
+        assert all(float(v[3]) > 0 for v in vendor) and all(float(v[3]) > 0 for v in ours)
+        assert len(diffs) == len(shapes)
+        for (m, n, k), (diff, largest) in zip(shapes, diffs):
+            # both are fp32 sums of the same exact products in different orders
+            assert float(diff) <= 2.0 * k * 2.0 ** -24 * float(largest) + 1e-6
+
+    check(run(5, 256, 512, 256), [(256, 256, 256), (512, 512, 512)])
+    check(run(5, "shape", 16, 1024, 512), [(16, 512, 1024)])
+    assert subprocess.run([exe], capture_output=True, text=True).returncode == 1      # usage
