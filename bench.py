@@ -96,7 +96,7 @@ class BoardSampler(threading.Thread):
                         digits = "".join(ch for ch in line.split(":")[1] if ch.isdigit())
                         if digits:
                             self.sclk_mhz.append(int(digits))
-            time.sleep(0.02)
+            time.sleep(0.005)
 
     def summary(self):
         cap = None
@@ -108,7 +108,7 @@ class BoardSampler(threading.Thread):
             return {"available": False}
         out = {"available": True, "samples": max(len(self.power_w), len(self.sclk_mhz)), "power_cap_w": cap}
         if self.power_w:
-            out.update(power_w_last=self.power_w[-1], power_w_max=max(self.power_w))
+            out.update(power_w_last=self.power_w[-1], power_w_max=max(self.power_w), power_w_median=statistics.median(self.power_w))
         if self.sclk_mhz:
             out.update(shader_clock_mhz_last=self.sclk_mhz[-1], shader_clock_mhz_median=statistics.median(self.sclk_mhz),
                        shader_clock_mhz_nominal=2400)
@@ -158,7 +158,7 @@ def time_launches(torch, fn, steps, warmup):
     return e0.elapsed_time(e1) / steps, wall_ms / steps
 
 
-LLM_SHAPES = [(n, k, m) for (n, k) in [(28672, 8192), (8192, 28672), (10240, 8192)] for m in (1, 16, 64, 256)]
+FMT_NAME = {0: "e4m3", 1: "e5m2"}
 
 
 def main():
@@ -169,6 +169,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host CPU leg")
     ap.add_argument("--no-vendor", action="store_true", help="skip the hipBLASLt comparison (a child process)")
     ap.add_argument("--no-llm-shapes", action="store_true", help="time only M=16 N=28672 K=8192 of the skinny shapes")
+    ap.add_argument("--no-more-shapes", action="store_true",
+                    help="skip 16384^3, the four pairings at 4096^3 and the K=32768 stress shapes")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel that FETCH_SIZE / WRITE_SIZE "
                          "counter readings are scaled by when this script runs under rocprofv3 --pmc")
@@ -196,15 +198,43 @@ def main():
     L = pkg.lib()
     stream = torch.cuda.current_stream().cuda_stream      # events and launches share this stream
 
-    def raw_launch(m, k, n, a, b, c):
+    def raw_launch(m, k, n, a, b, c, fa=0, fb=0):
         """The bare C-ABI call (a few microseconds of host time, so short kernels stay back to back)."""
         pa, pb, pc = a.data_ptr(), b.data_ptr(), c.data_ptr()
 
         def go(_i):
-            code = L.fp8gemm_launch(m, k, n, pa, 0, pb, 0, pc, 2, stream)
+            code = L.fp8gemm_launch(m, k, n, pa, fa, pb, fb, pc, 2, stream)
             if code != 0:
                 pkg.check(code)
         return go
+
+    def time_settled(m, k, n, fa, fb, A_host, B_host, steps, rows):
+        """One more BASELINE shape through fp8gemm_launch: operands to HBM, clocks settled under
+        this shape's own load, `steps` timed launches, a sample of full rows against the CPU
+        oracle (checker only).  Returns the record for the JSON line."""
+        dA = torch.from_numpy(A_host).to(dev)
+        dB = torch.from_numpy(B_host).to(dev)
+        dC = torch.empty((m, n), dtype=torch.float32, device=dev)
+        fn = raw_launch(m, k, n, dA, dB, dC, fa, fb)
+        settle(torch, fn)
+        ms_, _ = time_launches(torch, fn, steps, 5)
+        tf = 2.0 * m * n * k / (ms_ * 1e-3) / 1e12
+        rec = {"M": m, "N": n, "K": k, "a": FMT_NAME[fa], "b": FMT_NAME[fb], "steps": steps, "ms": ms_, "tflops": tf,
+               "frac_of_fp8_peak": tf / PEAK_FP8_TFLOPS, "plan": list(pkg.plan(m, k, n))}
+        try:
+            oracle = load_oracle()
+            ridx = np.asarray(rows, dtype=np.int32)
+            got = dC[torch.from_numpy(ridx).long().to(dev)].cpu().numpy()
+            ref, S = oracle.gemm(A_host, fa, B_host, fb, rows=ridx, with_scale=True)
+            err = np.abs(got.astype(np.float64) - ref)
+            tol = oracle.tolerance(k, S)
+            rec["parity"] = {"rows_checked": int(ridx.size), "worst_err_over_tol": float((err / tol).max()),
+                             "pass": bool(np.isfinite(got).all() and (err <= tol).all())}
+        except Exception as ex:
+            rec["parity"] = {"error": str(ex)[:200]}
+        del dA, dB, dC
+        torch.cuda.empty_cache()
+        return rec
 
     # ---------------------------------------------------------------- square, compute-bound
     M = N = K = 8192
@@ -229,6 +259,14 @@ def main():
     repeat_ms = [time_block(torch, go, args.steps) for _ in range(5)]
     sampler.stop_flag.set()
     sampler.join()
+    # board power and shader clock over one more second of the same launches, sampled every 5 ms
+    board_sampler = BoardSampler()
+    board_sampler.start()
+    t_board = time.perf_counter()
+    while time.perf_counter() - t_board < 1.0:
+        time_block(torch, go, 50)
+    board_sampler.stop_flag.set()
+    board_sampler.join()
     tflops = to_tflops(ms)
 
     # parity on a sample of full rows, against the CPU oracle (checker only)
@@ -261,6 +299,26 @@ def main():
                      "tflops": to_tflops(zero_ms), "frac_of_fp8_peak": to_tflops(zero_ms) / PEAK_FP8_TFLOPS,
                      "board": zero_sampler.summary()}
     del A, B, C
+    torch.cuda.empty_cache()
+
+    # ---------------------------------------------------------------- the other compute-bound BASELINE shapes
+    # (each through fp8gemm_launch, clocks settled under its own load; `value` stays the 8192^3 figure)
+    square_sweep = [{"M": M, "N": N, "K": K, "a": "e4m3", "b": "e4m3", "steps": args.steps, "ms": ms, "tflops": tflops,
+                     "frac_of_fp8_peak": tflops / PEAK_FP8_TFLOPS, "plan": list(pkg.plan(M, K, N)), "parity": parity}]
+    pairings_4096, stress_k32768 = [], []
+    if not args.no_more_shapes:
+        n16 = 16384
+        square_sweep.append(time_settled(
+            n16, n16, n16, 0, 0, pkg.fill((n16, n16), pkg.E4M3, seed=0xA11CE + 3, dist="normal"),
+            pkg.fill((n16, n16), pkg.E4M3, seed=0xB0B + 3, dist="normal"), max(10, args.steps // 5), [0, 255, 256, 8191, 16383]))
+        for fa, fb in [(0, 0), (1, 1), (0, 1), (1, 0)]:
+            pairings_4096.append(time_settled(
+                4096, 4096, 4096, fa, fb, pkg.fill((4096, 4096), fa, seed=0xA11CE + 2, dist="normal", sigma=4.0),
+                pkg.fill((4096, 4096), fb, seed=0xB0B + 2, dist="normal", sigma=4.0), args.steps, [0, 129, 1000, 2047, 4095]))
+        for fa, fb in [(1, 0), (0, 1)]:
+            stress_k32768.append(time_settled(
+                4096, 32768, 4096, fa, fb, pkg.fill((4096, 32768), fa, seed=0xA11CE + 5, dist="loguniform"),
+                pkg.fill((4096, 32768), fb, seed=0xB0B + 5, dist="loguniform"), max(10, args.steps // 2), [0, 1027, 4095]))
 
     # ---------------------------------------------------------------- LLM-linear shapes, HBM-bound
     # Cold figures: every launch reads a weight buffer that has been pushed out of the 256 MB
@@ -428,7 +486,9 @@ def main():
                        "frac_of_fp8_peak": to_tflops(settle_blocks[0]) / PEAK_FP8_TFLOPS},
         "repeats": {"what": "five more blocks of `steps` launches right after the timed one",
                     "tflops_median": rep_tf[2], "tflops_min": rep_tf[0], "tflops_max": rep_tf[-1]},
-        "board": sampler.summary(),
+        "board": dict(board_sampler.summary(), what="one more second of back-to-back launches of the same shape right after "
+                                                    "the timed ones, sysfs sampled every 5 ms",
+                      during_timed_steps=sampler.summary()),
         "zero_operands": zero_operands,
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / PEAK_FP8_TFLOPS, "traffic": TRAFFIC_BYTES_8192,
@@ -438,6 +498,9 @@ def main():
                                           TRAFFIC_8192["write_kib"], TRAFFIC_8192["write_scale"]),
                      "algorithmic_flops": flops, "algorithmic_bytes": alg_bytes,
                      "kernel_ms": ms},
+        "square_sweep": square_sweep,
+        "pairings_4096": pairings_4096,
+        "stress_k32768": stress_k32768,
         "skinny": skinny,
         "llm_shapes": llm,
         "parity": parity,

@@ -41,12 +41,10 @@ extern "C" {
  * of the reference's launch API (GEMM/include/gemm.cuh), argument order
  * (m, k, n, a, b, out) as there, default stream as there
  * (GEMM/src/gemm.cu:263-285).  "stage2" backs gemm::GEMM, "stage4" backs
- * gemm::GEMM4; the stage count selects the LDS pipeline depth of the tiled
- * kernel (2- and 3-deep rings of 128-byte K tiles, or 4-deep rings of 64-byte
- * ones) and never changes the result's contract.  Where the planned kernel
- * computes with the 16x16x128 MFMA, one MFMA step consumes 128 bytes of K, a
- * 4-deep ring of 64-byte K tiles and a 2-deep ring of 128-byte ones are the
- * same pipeline, and both stage counts run the same kernel.
+ * gemm::GEMM4.  Both run the same plan and the same kernels, as the reference's
+ * GEMM4 runs the kernel of GEMM (GEMM/src/gemm.cu:687-694): the depth of the LDS
+ * ring (2 to 5 slots) belongs to the tile shape that the planner picks for the
+ * problem, not to the entry point.
  */
 int fp8gemm_e4m3_e4m3_stage2(int m, int k, int n, const void *a, const void *b, float *out); /* gemm.cuh:12-15 */
 int fp8gemm_e4m3_e4m3_stage4(int m, int k, int n, const void *a, const void *b, float *out); /* gemm.cuh:18-21 */
@@ -176,8 +174,8 @@ int fp8gemm_tile_order(int m, int k, int n, int bm, int bn, int index, int *tile
 /*
  * Device scratch.  A shape whose plan cuts K into slices needs device memory for the
  * slices' partial sums; fp8gemm_scratch_bytes tells how much (0 when the shape needs
- * none: 8192^3, M=16 N=28672 K=8192, ...; the figure is for the stage-2 plan, the stage-4
- * plan cuts K the same way; it includes 16 KiB of arrival counters ahead of the sums).
+ * none: 8192^3, M=16 N=28672 K=8192, ...; the same for both stage counts, which run the same
+ * plan; it includes 16 KiB of arrival counters ahead of the sums).
  * With the library's own scratch the slices of tiles up to 128 x 128 are added up inside the
  * GEMM kernel, by the slice of a tile that arrives last (the counters start at zero and
  * every kernel leaves them at zero); larger tiles, and every shape run on a caller's

@@ -16,22 +16,13 @@ namespace fp8gemm_detail {
 
 // ------------------------------------------------------------------ variants
 // Tiled kernel shapes: <BM, BN, BK, waves_m, waves_n, stages, swizzle>.
-using TileP2 = TileShape<256, 256, 128, 2, 2, 2, 3>;  // persistent, 2 x 64 KiB ring, 128x128 per wave
+using TileP2 = TileShape<256, 256, 128, 2, 2, 2, 3>;  // 2 x 64 KiB ring, 128x128 per wave
 using TileP2h = TileShape<256, 256, 128, 2, 2, 2, 3, true>;   // the same on v_mfma_f32_16x16x128_f8f6f4
 using TileT2h = TileShape<192, 256, 128, 2, 2, 2, 3, true>;   // 192 x 256 on that MFMA
-using TileP4 = TileShape<256, 256, 64, 2, 2, 4, 2>;   // persistent, 4 x 32 KiB ring
-using TileP8 = TileShape<256, 256, 128, 2, 4, 2, 3>;  // persistent, 8 waves, 128x64 per wave
-using TileS2 = TileShape<128, 128, 128, 2, 2, 2, 3>;  // one tile per workgroup, for small problems
-using TileS4 = TileShape<128, 128, 128, 2, 2, 4, 3>;
-using TileH3 = TileShape<128, 256, 128, 2, 2, 3, 3>;  // persistent, half-height tile, 3 x 48 KiB ring
-using TileQ2 = TileShape<128, 128, 128, 2, 2, 2, 3>;  // persistent, quarter tile
-using TileS64 = TileShape<128, 128, 64, 2, 2, 4, 2>;  // one tile per workgroup, 64-byte K tiles
-using TileW3 = TileShape<256, 128, 128, 2, 2, 3, 3>;  // persistent, half-width tile, 3 x 48 KiB ring
-using TileT2 = TileShape<192, 256, 128, 2, 2, 2, 3>;  // persistent, three-quarter-height tile: other tile counts
-// the 4-deep rings of 64-byte K tiles behind the stage-4 entry points, same tile shapes
-using TileT4 = TileShape<192, 256, 64, 2, 2, 4, 2>;
-using TileH4 = TileShape<128, 256, 64, 2, 2, 4, 2>;
-using TileQ4 = TileShape<128, 128, 64, 2, 2, 4, 2>;
+using TileH3 = TileShape<128, 256, 128, 2, 2, 3, 3>;  // half-height tile, 3 x 48 KiB ring
+using TileQ2 = TileShape<128, 128, 128, 2, 2, 2, 3>;  // quarter tile
+using TileW3 = TileShape<256, 128, 128, 2, 2, 3, 3>;  // half-width tile, 3 x 48 KiB ring
+using TileT2 = TileShape<192, 256, 128, 2, 2, 2, 3>;  // three-quarter-height tile: other tile counts
 // weight streaming through the tiled kernel (one row of tiles, B read once with the non-temporal hint):
 // deep rings, so that many bytes of B are in flight per CU
 // (M=64 N=28672 K=8192, weights cold: 39.3 us against 50.0 us of the single-wave streaming kernel; rings of 4, 5
@@ -44,10 +35,6 @@ template <int MT, int TN>
 using SkinnyV0 = SkinnyShape<MT, TN, 128, 5>;
 template <int MT, int TN>
 using SkinnyV1 = SkinnyShape<MT, TN, 256, 4>;
-template <int MT, int TN>
-using SkinnyV2 = SkinnyShape<MT, TN, 128, 8>;
-template <int MT, int TN>
-using SkinnyV3 = SkinnyShape<MT, TN, 256, 6>;
 template <int MT, int TN>
 using SkinnyV4 = SkinnyShape<MT, TN, 512, 4, 80 * 1024>;
 template <int MT, int TN>
@@ -72,8 +59,6 @@ hipError_t allow_lds(Kernel kernel, int bytes)
     return e;
 }
 
-template <class S, int AF, int BF>
-struct TileKernelTag {};
 template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM>
 struct PtileKernelTag {};
 template <class S, int AF, int BF>
@@ -92,28 +77,6 @@ hipError_t launch_direct(int m, int k, int n, const uint8_t *a, const uint8_t *b
 }
 
 // ------------------------------------------------------------------ tiled
-template <class S, int AF, int BF>
-hipError_t launch_tile_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, float *out,
-                             hipStream_t stream)
-{
-    if (k % S::BK != 0) return hipErrorInvalidValue;
-    const int tiles_m = (m + S::BM - 1) / S::BM;
-    const int tiles_n = (n + S::BN - 1) / S::BN;
-    // XCD-local super-blocks of tiles: 32 CUs per XCD -> blocks of up to 32 tiles,
-    // shaped to balance A-panel and B-panel reuse.
-    int GM = 4, GN = 8;
-    if (tiles_m < GM) { GM = tiles_m; }
-    if (tiles_n < GN) { GN = tiles_n; }
-    const int nb = ((tiles_m + GM - 1) / GM) * ((tiles_n + GN - 1) / GN);
-    const long grid = (long)((nb + 7) / 8) * 8 * GM * GN;
-    auto kernel = gemm_tile_kernel<S, AF, BF>;
-    hipError_t e = allow_lds<TileKernelTag<S, AF, BF>>(kernel, S::LDS_BYTES);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(S::THREADS), S::LDS_BYTES, stream,
-                       m, k, n, a, b, out, tiles_m, tiles_n, GM, GN);
-    return hipGetLastError();
-}
-
 // Start skew between the tile rows of an XCD's window, in ticks of 10 ns (see the kernel).  It
 // costs three times the skew once and shortens every epilogue (8192^3: 368 -> 365 us with 1.5 to
 // 2.5 us, 375 us with 4 us), so it is used from four rounds of whole tiles on.
@@ -162,7 +125,9 @@ hipError_t launch_ptile_shape_k(int m, int k, int n, const uint8_t *a, const uin
         if (e != hipSuccess) return e;
         base = static_cast<float *>(p);
         ws = base + kSliceCounterBytes / sizeof(float);
-        if (kSumInKernel && wsp.counters_zero() && w.tail <= kMaxSliceCounters) counters = static_cast<int *>(p);
+        // (the kernel addresses the partial sums through a buffer window with 32-bit offsets)
+        const bool window_fits = ptile_scratch_bytes(w, S::BM, S::BN) <= 0xFFFFFFFFull;
+        if (kSumInKernel && wsp.counters_zero() && w.tail <= kMaxSliceCounters && window_fits) counters = static_cast<int *>(p);
     }
     hipError_t e;
     if constexpr (STREAM_TOO && !KOVER) {
@@ -202,24 +167,12 @@ template <int AF, int BF>
 hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
                        int variant, int nsplit, bool split_all, int rotate, const OutSpec &spec, Workspace &wsp, hipStream_t stream)
 {
-    const bool persistent = !(variant == 3 || variant == 4 || variant == 7);
-    if (!persistent && nsplit != 1) return hipErrorInvalidValue;   // K slices only in the persistent kernels
-    // the one-tile-per-workgroup kernels write bare fp32 sums only
-    if (!persistent && !plain_output(spec)) return hipErrorInvalidValue;
     switch (variant) {
     case 0: return launch_ptile_shape<TileP2, AF, BF, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
-    case 1: return launch_ptile_shape<TileP4, AF, BF, true, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
-    case 2: return launch_ptile_shape<TileP8, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
-    case 3: return launch_tile_shape<TileS2, AF, BF>(m, k, n, a, b, static_cast<float *>(out), stream);
-    case 4: return launch_tile_shape<TileS4, AF, BF>(m, k, n, a, b, static_cast<float *>(out), stream);
     case 5: return launch_ptile_shape<TileH3, AF, BF, true, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
     case 6: return launch_ptile_shape<TileQ2, AF, BF, true, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
-    case 7: return launch_tile_shape<TileS64, AF, BF>(m, k, n, a, b, static_cast<float *>(out), stream);
     case 8: return launch_ptile_shape<TileW3, AF, BF, false, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
     case 9: return launch_ptile_shape<TileT2, AF, BF, false, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
-    case 10: return launch_ptile_shape<TileT4, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
-    case 11: return launch_ptile_shape<TileH4, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
-    case 12: return launch_ptile_shape<TileQ4, AF, BF, false, false>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
     case 13:
         if (!p2h_ok(k, nsplit)) return hipErrorInvalidValue;
         return launch_ptile_shape<TileP2h, AF, BF, true, true>(m, k, n, a, b, out, nsplit, split_all, rotate, spec, wsp, stream);
@@ -266,9 +219,6 @@ hipError_t launch_skinny_mt(int m, int k, int n, const uint8_t *a, const uint8_t
 #define SK(MT, TN) \
     if (p.mt == MT && p.tn == TN) return launch_skinny_shape<V<MT, TN>, AF, BF>(m, k, n, a, b, out, p.nsplit, spec, wsp, stream);
     SK(1, 1) SK(1, 2) SK(1, 4)
-    SK(2, 1) SK(2, 2) SK(2, 4)
-    SK(3, 1) SK(3, 2) SK(3, 4)
-    SK(4, 1) SK(4, 2) SK(4, 4)
 #undef SK
     return hipErrorInvalidValue;
 }
@@ -280,8 +230,6 @@ hipError_t launch_skinny(int m, int k, int n, const uint8_t *a, const uint8_t *b
     switch (p.variant) {
     case 0: return launch_skinny_mt<SkinnyV0, AF, BF>(m, k, n, a, b, out, p, spec, wsp, stream);
     case 1: return launch_skinny_mt<SkinnyV1, AF, BF>(m, k, n, a, b, out, p, spec, wsp, stream);
-    case 2: return launch_skinny_mt<SkinnyV2, AF, BF>(m, k, n, a, b, out, p, spec, wsp, stream);
-    case 3: return launch_skinny_mt<SkinnyV3, AF, BF>(m, k, n, a, b, out, p, spec, wsp, stream);
     case 4: return launch_skinny_mt<SkinnyV4, AF, BF>(m, k, n, a, b, out, p, spec, wsp, stream);
     case 5: return launch_skinny_mt<SkinnyV5, AF, BF>(m, k, n, a, b, out, p, spec, wsp, stream);
     default: return hipErrorInvalidValue;
@@ -289,7 +237,7 @@ hipError_t launch_skinny(int m, int k, int n, const uint8_t *a, const uint8_t *b
 }
 
 template <int AF, int BF>
-hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out, int stages,
+hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
                     int algo, int variant, int nsplit, const OutSpec &spec, Workspace &wsp, hipStream_t stream)
 {
     const bool aligned = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) % 16) == 0;
@@ -302,7 +250,7 @@ hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, voi
         return launch_direct<AF, BF>(m, k, n, a, b, out, spec, stream);
     case FP8GEMM_ALGO_TILE: {
         if (!aligned || k % 16 != 0 || k > (1 << 23)) return hipErrorInvalidValue;
-        TilePlan p = plan_tile(m, k, n, stages);
+        TilePlan p = plan_tile(m, k, n);
         if (variant >= 0) {
             // tuning hook: variant = shape index + 16 * (1 + K-walk rotation mode); a bare
             // shape index keeps the plan's rotation and runs unsplit unless split_k says otherwise

@@ -19,13 +19,13 @@
 
 namespace fp8gemm_detail {
 
-extern template hipError_t dispatch<0, 0>(int, int, int, const uint8_t *, const uint8_t *, void *, int, int, int, int,
+extern template hipError_t dispatch<0, 0>(int, int, int, const uint8_t *, const uint8_t *, void *, int, int, int,
                                           const OutSpec &, Workspace &, hipStream_t);
-extern template hipError_t dispatch<0, 1>(int, int, int, const uint8_t *, const uint8_t *, void *, int, int, int, int,
+extern template hipError_t dispatch<0, 1>(int, int, int, const uint8_t *, const uint8_t *, void *, int, int, int,
                                           const OutSpec &, Workspace &, hipStream_t);
-extern template hipError_t dispatch<1, 0>(int, int, int, const uint8_t *, const uint8_t *, void *, int, int, int, int,
+extern template hipError_t dispatch<1, 0>(int, int, int, const uint8_t *, const uint8_t *, void *, int, int, int,
                                           const OutSpec &, Workspace &, hipStream_t);
-extern template hipError_t dispatch<1, 1>(int, int, int, const uint8_t *, const uint8_t *, void *, int, int, int, int,
+extern template hipError_t dispatch<1, 1>(int, int, int, const uint8_t *, const uint8_t *, void *, int, int, int,
                                           const OutSpec &, Workspace &, hipStream_t);
 
 namespace {
@@ -203,32 +203,24 @@ bool p2h_ok(int k, int nsplit)
     return k % 16 == 0 && ((k + 127) / 128) / nsplit >= 2;
 }
 
-// the single-wave streams, up to 64 rows
+// the single-wave streams: up to 16 rows of A (one 16-row MFMA block)
 bool skinny_ok(int m, int k, int n)
 {
-    return m <= 64 && n % 16 == 0 && k % 128 == 0;
+    return m <= 16 && n % 16 == 0 && k % 128 == 0;
 }
 
 // Picks columns per wave, LDS shape and split-K factor.  Measured on MI355X with
-// operands that are cold in every cache.  Up to 32 rows of A the HBM pipe is fullest
-// with one to two fat streams per CU (256..512 streams, each with a deep LDS ring)
-// rather than many thin ones, and a split-K pass costs 10 % and more, so K is cut only
-// when the columns alone give too few streams.  From 33 rows on a stream spends most
-// of its LDS ring on A: the widest column group (64 columns) keeps the share of B up,
-// and about two streams per CU hide the longer MFMA phases, even at the price of K
-// slices.  Long K steps (512 bytes per row and load group) help a little.
+// operands that are cold in every cache.  The HBM pipe is fullest with one to two fat
+// streams per CU (256..512 streams, each with a deep LDS ring) rather than many thin
+// ones, and a split-K pass costs 10 % and more, so K is cut only when the columns alone
+// give too few streams.
 SkinnyPlan plan_skinny(int m, int k, int n)
 {
     SkinnyPlan p;
-    p.mt = (m + 15) / 16;
+    p.mt = 1;
     const int ksteps = k / 128;
     int tn = 4, split = 1;
-    if (p.mt >= 3) {
-        while (n % (16 * tn) != 0) tn /= 2;       // n % 16 == 0 is guaranteed by the caller
-        // slices shorter than 4 KiB of K lose more to their ramp than the extra streams gain
-        while ((long)(n / (16 * tn)) * split < 448 && split < 16 && ksteps % (2 * split) == 0 && ksteps / (2 * split) >= 32)
-            split *= 2;
-    } else {
+    {
         // Streams of 64, 32 or 16 columns: the widest that still gives 400 streams or more (every
         // stream re-reads A, and a wide stream's ring holds more of B per load instruction); with
         // more than a few rows of A, a count that fills the 256 CUs evenly (a multiple of 256) is
@@ -268,7 +260,7 @@ SkinnyPlan plan_skinny(int m, int k, int n)
     // longer K steps, so that a ring stage still holds 16 KiB or more: the thinnest, on a long K
     // and with two waves or more per CU, whole 1 KiB rows.  Three waves or more per CU on a
     // short K: a ring small enough for all of them to be resident at once.
-    if (tn == 4 && p.mt <= 3)
+    if (tn == 4)
         p.variant = 0;
     else if (tn == 1 && kchunk % 1024 == 0 && kchunk >= 8192 && waves >= 512)
         p.variant = 5;
@@ -285,7 +277,7 @@ SkinnyPlan plan_skinny(int m, int k, int n)
 // re-reads all of A for every 64 columns.
 int select_algo(int m, int k, int n)
 {
-    if (skinny_ok(m, k, n) && m <= 16) return FP8GEMM_ALGO_SKINNY;
+    if (skinny_ok(m, k, n)) return FP8GEMM_ALGO_SKINNY;
     if (k % 16 == 0 && k <= (1 << 23)) return FP8GEMM_ALGO_TILE;
     return FP8GEMM_ALGO_DIRECT;
 }
@@ -301,32 +293,34 @@ int select_algo(int m, int k, int n)
 //   K slices add one reduction pass over (nsplit + 1) x the cut tiles.
 // The model only has to rank the candidates, not to predict the time.
 struct PtileCost {
-    int variant, variant4, bm, bn;              // variant4: the same tile with a 4-deep ring of 64-byte K tiles (-1: none)
+    int variant, bm, bn;
     double per_k_tile, per_item, stream_rate;   // us, us, bytes per us
 };
 constexpr PtileCost kPtileCosts[] = {
-    {0, 1, 256, 256, 1.30, 13.0, 4.0e6},
-    {13, 13, 256, 256, 1.25, 13.0, 4.0e6},     // the same tile on the 16x16x128 MFMA: less energy per flop, and
-                                               // the compute-bound shapes run at the board's power limit.  One MFMA
-                                               // step takes 128 bytes of K, so a 4-deep ring of 64-byte K tiles and
-                                               // a 2-deep ring of 128-byte ones are the same pipeline: the 4-stage
-                                               // entry points share this kernel with the 2-stage ones
-    {9, 10, 192, 256, 1.15, 9.0, 4.6e6},
-    {14, 14, 192, 256, 1.10, 9.0, 4.0e6},
-    {5, 11, 128, 256, 1.00, 6.0, 6.5e6},
-    {6, 12, 128, 128, 0.75, 2.5, 4.0e6},
-    {8, -1, 256, 128, 0.90, 10.0, 4.6e6},
-    // weight streaming (one row of tiles, B loaded once with the non-temporal hint, deep rings); their rings
-    // are 5 and 4 slots deep, so the 4-stage entry points run them too
-    {15, 15, 64, 128, 0.586, 5.5, 6.4e6},
-    {16, 16, 128, 128, 0.70, 5.5, 6.0e6},
+    {0, 256, 256, 1.30, 13.0, 4.0e6},
+    {13, 256, 256, 1.25, 13.0, 4.0e6},         // the same tile on the 16x16x128 MFMA: less energy per flop, and
+                                               // the compute-bound shapes run at the board's power limit
+    {9, 192, 256, 1.15, 9.0, 4.6e6},
+    {14, 192, 256, 1.10, 9.0, 4.0e6},
+    {5, 128, 256, 1.00, 6.0, 6.5e6},
+    {6, 128, 128, 0.75, 2.5, 4.0e6},
+    {8, 256, 128, 0.90, 10.0, 4.6e6},
+    // weight streaming (one row of tiles, B loaded once with the non-temporal hint, rings 5 and 4 slots deep)
+    {15, 64, 128, 0.586, 5.5, 6.4e6},
+    {16, 128, 128, 0.70, 5.5, 6.0e6},
 };
 constexpr double kIdleChipFactor = 0.6;
 constexpr int kSplitChoices[] = {1, 2, 3, 4, 6, 8, 12, 16};
 constexpr int kMinKTilesPerSlice = 12;
 constexpr size_t kMaxSplitScratch = (size_t)1 << 30;
 
-TilePlan plan_tile(int m, int k, int n, int stages)
+// The plan does not depend on the stage count of the entry point: the depth of the LDS ring (2 to
+// 5 slots) belongs to the tile shape, and the 2- and 4-stage entry points run the same kernels --
+// as the reference's GEMM4 runs the kernel of GEMM (GEMM/src/gemm.cu:687-694).  On the 16x16x128
+// MFMA, whose one step takes 128 bytes of K, a 4-deep ring of 64-byte K tiles and a 2-deep ring of
+// 128-byte ones are the same pipeline; 4-deep rings of 64-byte K tiles under the 32x32x64 MFMA
+// measured 5 to 11 % slower than the 2- and 3-deep rings of 128-byte K tiles on every shape class.
+TilePlan plan_tile(int m, int k, int n)
 {
     TilePlan best = {0, 1, 2, false};
     const int kt = (k + 127) / 128;
@@ -339,14 +333,8 @@ TilePlan plan_tile(int m, int k, int n, int stages)
         if ((c.variant == 15 || c.variant == 16) && (m > c.bm || k % 128 != 0)) continue;
         // ... and up to 64 rows nothing else comes close to them
         if (m <= 64 && k % 128 == 0 && c.variant != 15) continue;
-        if (stages == 4) {
-            // the 4-deep rings rank like their 2- and 3-deep twins (same tiles, same work list);
-            // only the 256 x 256 one (and the 16x16x128 kernels they share with the 2-stage entry
-            // points) is compiled for a K that is not a multiple of its K tile
-            if (c.variant4 < 0 || (k % 64 != 0 && !(c.variant4 == 1 || c.variant4 == 13 || c.variant4 == 14))) continue;
-        } else if (k % 128 != 0 && !(c.variant == 0 || c.variant == 5 || c.variant == 6 || c.variant == 13 || c.variant == 14)) {
-            continue;      // overhanging K tile: only the shapes compiled for it
-        }
+        // overhanging K tile: only the shapes compiled for it
+        if (k % 128 != 0 && !(c.variant == 0 || c.variant == 5 || c.variant == 6 || c.variant == 13 || c.variant == 14)) continue;
         for (int mode = 0; mode < 2; ++mode)          // 0: slices for the tail tiles only, 1: for all
             for (int split : kSplitChoices) {
                 if (mode == 1 && split == 1) continue;      // same as mode 0
@@ -371,7 +359,7 @@ TilePlan plan_tile(int m, int k, int n, int stages)
                 if (w.nsplit > 1) cost += 6.0 + (w.nsplit + 1) * (double)w.tail * c.bm * c.bn * 4.0 / 6.0e6;
                 if (cost < best_cost) {
                     best_cost = cost;
-                    best.variant = stages == 4 ? c.variant4 : c.variant;
+                    best.variant = c.variant;
                     best.nsplit = w.nsplit;
                     best.split_all = mode == 1;
                 }
@@ -387,7 +375,7 @@ size_t tile_plan_scratch_bytes(int m, int n, const TilePlan &p)
 {
     if (p.nsplit <= 1) return 0;
     for (const PtileCost &c : kPtileCosts)
-        if (c.variant == p.variant || c.variant4 == p.variant) {
+        if (c.variant == p.variant) {
             const PtileWork w = ptile_work(m, n, c.bm, c.bn, p.nsplit, p.split_all);
             return w.ok ? ptile_scratch_bytes(w, c.bm, c.bn) : 0;
         }
@@ -415,13 +403,13 @@ int launch_checked(int m, int k, int n, const void *a, int a_fmt, const void *b,
     (void)hipGetLastError();
     hipError_t e;
     if (a_fmt == FP8GEMM_E4M3 && b_fmt == FP8GEMM_E4M3)
-        e = dispatch<0, 0>(m, k, n, pa, pb, out, stages, algo, variant, nsplit, spec, wsp, s);
+        e = dispatch<0, 0>(m, k, n, pa, pb, out, algo, variant, nsplit, spec, wsp, s);
     else if (a_fmt == FP8GEMM_E5M2 && b_fmt == FP8GEMM_E5M2)
-        e = dispatch<1, 1>(m, k, n, pa, pb, out, stages, algo, variant, nsplit, spec, wsp, s);
+        e = dispatch<1, 1>(m, k, n, pa, pb, out, algo, variant, nsplit, spec, wsp, s);
     else if (a_fmt == FP8GEMM_E4M3)
-        e = dispatch<0, 1>(m, k, n, pa, pb, out, stages, algo, variant, nsplit, spec, wsp, s);
+        e = dispatch<0, 1>(m, k, n, pa, pb, out, algo, variant, nsplit, spec, wsp, s);
     else
-        e = dispatch<1, 0>(m, k, n, pa, pb, out, stages, algo, variant, nsplit, spec, wsp, s);
+        e = dispatch<1, 0>(m, k, n, pa, pb, out, algo, variant, nsplit, spec, wsp, s);
     return (int)e;
 }
 
@@ -576,7 +564,7 @@ int fp8gemm_plan(int m, int k, int n, int stages, int plan[4])
         plan[2] = p.nsplit;
         plan[3] = 16 * p.tn;
     } else if (algo == FP8GEMM_ALGO_TILE) {
-        const TilePlan p = plan_tile(m, k, n, stages);
+        const TilePlan p = plan_tile(m, k, n);
         plan[1] = p.variant;
         plan[2] = p.nsplit;
         plan[3] = p.rotate + ((p.nsplit > 1 && !p.split_all) ? 16 : 0);
@@ -599,7 +587,7 @@ size_t fp8gemm_scratch_bytes(int m, int k, int n)
     int nsplit = 1;
     const int algo = select_algo(m, k, n);
     if (algo == FP8GEMM_ALGO_SKINNY) nsplit = plan_skinny(m, k, n).nsplit;
-    if (algo == FP8GEMM_ALGO_TILE) return tile_plan_scratch_bytes(m, n, plan_tile(m, k, n, 2));
+    if (algo == FP8GEMM_ALGO_TILE) return tile_plan_scratch_bytes(m, n, plan_tile(m, k, n));
     return nsplit > 1 ? kSliceCounterBytes + (size_t)nsplit * m * n * sizeof(float) : 0;
 }
 

@@ -28,7 +28,7 @@
 // registers of a lane are then 4 consecutive columns of one row of C, which
 // turns the epilogue into 128-bit stores.
 //
-// LDS layout, swizzle and the K-permutation freedom are as in kernel_tile.h.
+// LDS layout, swizzle and the K-permutation freedom are described in kernel_tile.h.
 // Requirements checked by the host: K % 16 == 0 (rows start 16-byte aligned and a
 // 16-byte chunk never straddles the end of a row), K < 2^23, 16-byte aligned a and b.
 #ifndef FP8GEMM_KERNEL_PTILE_H
@@ -730,16 +730,23 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
             if (EX && finish) amax_commit(spec, amax_local);
         }
         // ---- K slices: the slice that arrives last adds them up ---------------------
-        // Every slice of a cut tile has written its partial sums to its scratch slot with
-        // device-scope stores.  Once those are done (the barrier waits for them) it counts
-        // itself on the tile's arrival counter, and the one that finds all the others there
-        // reads the slots back in slice order -- the order the reduction kernel uses, so the
-        // bits are the same -- and writes the tile of C.  Nobody waits for anybody.  The
-        // counter is left at zero for the next launch.
+        // Hand-over of the partial sums between workgroups that may sit on different XCDs, in
+        // three steps:
+        //   1. every thread writes its partial sums with device-scope (sc1) stores and waits for
+        //      them itself (s_waitcnt vmcnt(0)): such a store counts as done only once it is
+        //      written through.  A workgroup barrier does not wait for outstanding stores;
+        //   2. after the barrier (all threads' stores are done) one thread counts the slice on the
+        //      tile's arrival counter with a device-scope atomic;
+        //   3. the slice that finds all the others there reads the slots back with device-scope
+        //      (sc1) loads, issued only after the counter's value is known (they depend on it
+        //      through the flag in LDS and a barrier), in slice order -- the order the reduction
+        //      kernel uses, so the bits are the same -- and writes the tile of C.
+        // Nobody waits for anybody.  The counter is left at zero for the next launch.
         if (SUM_HERE && to_ws && counters) {                       // (uniform)
             const int t_cut = ws_slot % tail;                      // number of the cut tile
             LDS_AS int *flag = (LDS_AS int *)(lds + S::PTILE_LDS_BYTES + 256);
-            __syncthreads();                                       // (s_waitcnt vmcnt(0) ahead of the barrier)
+            wait_vmcnt<0>();                                       // step 1: this thread's stores are written through
+            __syncthreads();
             if (tid == 0) {
                 const int before = __hip_atomic_fetch_add(counters + t_cut, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 const int last = before == nsplit - 1;

@@ -14,8 +14,10 @@
 
 namespace fp8gemm_detail {
 
-// tiled kernel shapes: 0 P2, 1 P4, 2 P8, 3 S2, 4 S4, 5 H3, 6 Q2, 7 S64, 8 W3, 9 T2, 10 T4, 11 H4, 12 Q4, 13 P2h, 14 T2h,
-// 15 E5, 16 Q4s
+// Tiled kernel shapes by number (the tuning hook's `variant`): 0 P2 (256 x 256), 5 H3 (128 x 256), 6 Q2 (128 x 128),
+// 8 W3 (256 x 128), 9 T2 (192 x 256), 13 P2h and 14 T2h (256 x 256 and 192 x 256 on the 16x16x128 MFMA), 15 E5 (64 x 128,
+// weight streaming), 16 Q4s (128 x 128, weight streaming).  Streaming (single-wave) ring shapes: 0, 1, 4, 5.  A number
+// below the count that is not listed names no compiled kernel and is refused.
 constexpr int kNumTileVariants = 17;
 constexpr int kNumSkinnyVariants = 6;
 
@@ -53,7 +55,7 @@ struct TilePlan {
     int variant, nsplit, rotate;
     bool split_all;      // K slices for every tile (else only for the tiles that do not fill a round)
 };
-TilePlan plan_tile(int m, int k, int n, int stages);
+TilePlan plan_tile(int m, int k, int n);
 size_t tile_plan_scratch_bytes(int m, int n, const TilePlan &p);
 
 // Where the partial sums of one call's K slices go: a buffer of the per-(device, stream)
@@ -91,7 +93,7 @@ hipError_t launch_tile_slices_reduce(const float *ws, void *out, int m, int n, i
 // Validated operands -> kernel choice and launch for one operand pairing (AF, BF: 0 = E4M3,
 // 1 = E5M2).  Each pairing is compiled in a translation unit of its own (dispatch_pair.hip).
 template <int AF, int BF>
-hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out, int stages,
+hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
                     int algo, int variant, int nsplit, const OutSpec &spec, Workspace &wsp, hipStream_t stream);
 
 }  // namespace fp8gemm_detail

@@ -189,7 +189,11 @@ def test_plans_are_consistent_over_random_shapes(pkg):
         k = int(rng.integers(1, 260)) * int(rng.choice([16, 64, 128]))
         n = int(rng.integers(1, 1800)) * int(rng.choice([1, 16, 16, 128]))
         shapes.append((m, k, n))
+    compiled_tiles = {0, 5, 6, 8, 9, 13, 14, 15, 16}
+    compiled_streams = {0, 1, 4, 5}
     for (m, k, n) in shapes:
+        # the 2- and 4-stage entry points run the same plan (so one scratch figure serves both)
+        assert pkg.plan(m, k, n, 4) == pkg.plan(m, k, n, 2)
         for stages in (2, 4):
             fam, var, slices, extra = pkg.plan(m, k, n, stages)
             assert fam == L.fp8gemm_select_algo(m, k, n)
@@ -197,13 +201,13 @@ def test_plans_are_consistent_over_random_shapes(pkg):
             if fam == pkg.ALGO_SKINNY:
                 assert m <= 16 and k % 128 == 0 and n % 16 == 0
                 assert extra in (16, 32, 64) and n % extra == 0
-                assert 0 <= var < n_stream_variants
+                assert 0 <= var < n_stream_variants and var in compiled_streams
                 assert k % (128 * slices) == 0
                 if stages == 2:
                     want = COUNTERS + slices * m * n * 4 if slices > 1 else 0
                     assert L.fp8gemm_scratch_bytes(m, k, n) == want
             elif fam == pkg.ALGO_TILE:
-                assert k % 16 == 0 and 0 <= var < n_tile_variants
+                assert k % 16 == 0 and 0 <= var < n_tile_variants and var in compiled_tiles
                 assert slices == 1 or (k + 127) // 128 >= 2 * slices
                 if stages == 2:
                     need = L.fp8gemm_scratch_bytes(m, k, n)

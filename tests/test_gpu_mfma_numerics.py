@@ -24,7 +24,7 @@ FAMILIES = [
     ("tile 192x256 16x16x128", dict(algo=2, variant=14), 64),
     ("tile 128x256 3-deep", dict(algo=2, variant=5), 64),
     ("tile 128x128", dict(algo=2, variant=6), 64),
-    ("tile 256x256 4-deep 64-byte K tiles", dict(algo=2, variant=1), 64),
+    ("tile 192x256 32x32x64", dict(algo=2, variant=9), 64),
     ("tile 64x128 streaming", dict(algo=2, variant=15), 64),
 ]
 K = 256

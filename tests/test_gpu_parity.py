@@ -71,8 +71,8 @@ SHAPES = [
     ("direct", (40, 1030, 70)),
     ("tile", (128, 128, 128)), ("tile", (256, 384, 512)), ("tile", (300, 256, 200)), ("tile", (512, 1024, 768)),
     ("tile", (1, 128, 1)),
-    ("skinny", (16, 256, 64)), ("skinny", (1, 512, 128)), ("skinny", (13, 1024, 256)), ("skinny", (64, 512, 192)),
-    ("skinny", (33, 2048, 80)),
+    ("skinny", (16, 256, 64)), ("skinny", (1, 512, 128)), ("skinny", (13, 1024, 256)), ("skinny", (16, 512, 192)),
+    ("skinny", (5, 2048, 80)),
 ]
 
 
@@ -98,7 +98,7 @@ def test_all_finite_codes(pkg, oracle, fa, fb, algo, shape):
 @pytest.mark.parametrize("fa,fb", PAIRS)
 @pytest.mark.parametrize("algo,shape", [
     ("direct", (64, 2048, 96)), ("tile", (256, 2048, 256)), ("tile", (384, 4096, 640)),
-    ("skinny", (16, 4096, 512)), ("skinny", (64, 2048, 256)), ("skinny", (1, 8192, 256)),
+    ("skinny", (16, 4096, 512)), ("skinny", (9, 2048, 256)), ("skinny", (1, 8192, 256)),
     ("auto", (64, 4096, 1536)), ("auto", (33, 8192, 640)), ("auto", (17, 2048, 2048)), ("auto", (100, 4096, 1920)),
 ])
 def test_normal_inputs_within_fp32_reordering_bound(pkg, oracle, fa, fb, algo, shape):
@@ -113,12 +113,12 @@ def test_normal_inputs_within_fp32_reordering_bound(pkg, oracle, fa, fb, algo, s
 
 
 @pytest.mark.parametrize("fa,fb", PAIRS)
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 15, 16])
+@pytest.mark.parametrize("variant", [0, 5, 6, 8, 9, 15, 16])
 @pytest.mark.parametrize("shape", [(256, 256, 256), (300, 512, 200), (1000, 1024, 900), (513, 384, 257), (64, 128, 2048),
                                    (40, 640, 1000)])
 def test_every_tile_variant(pkg, oracle, variant, shape, fa, fb):
-    """Each compiled shape of the tiled kernels (persistent and one-tile-per-workgroup),
-    on shapes that overhang the tile in m and n, for all four pairings."""
+    """Each compiled shape of the tiled kernel on the 32x32x64 MFMA, on shapes that overhang
+    the tile in m and n, for all four pairings."""
     M, K, N = shape
     rng = np.random.default_rng(zlib.crc32(repr((variant, shape, fa, fb)).encode()))
     A = random_codes(rng, (M, K), fa)
@@ -178,7 +178,7 @@ def test_16x16x128_variant_refuses_a_single_k_tile(pkg, variant):
         run_gpu(pkg, A, 0, B, 0, algo=ALGOS["tile"], variant=variant)
 
 
-@pytest.mark.parametrize("variant,split", [(0, 2), (0, 3), (1, 5), (5, 4), (5, 7), (6, 2), (6, 16), (2, 2), (8, 3), (13, 2), (13, 4), (14, 3),
+@pytest.mark.parametrize("variant,split", [(0, 2), (0, 3), (9, 5), (5, 4), (5, 7), (6, 2), (6, 16), (8, 3), (13, 2), (13, 4), (14, 3),
                                            (15, 3), (15, 4), (16, 2)])
 @pytest.mark.parametrize("shape", [(256, 2048, 512), (300, 4096, 200), (1000, 2304, 900), (128, 8192, 2048)])
 def test_tile_k_slices(pkg, oracle, variant, split, shape):
@@ -200,7 +200,7 @@ def test_tile_k_slices(pkg, oracle, variant, split, shape):
     (5, -4, (2100, 1536, 4500)),      # 17 x 18 tiles of 128 x 256
     (0, -2, (4200, 1024, 4300)),      # 17 x 17 tiles of 256 x 256
     (8, -5, (4352, 1280, 2200)),      # 17 x 18 tiles of 256 x 128
-    (1, -2, (4352, 1088, 4352)),      # 64-byte K tiles, 17 of them
+    (9, -2, (3300, 1152, 4352)),      # 18 x 17 tiles of 192 x 256
 ])
 def test_tile_k_slices_for_the_last_partial_round(pkg, oracle, variant, split, shape):
     """More tiles than CUs: the rounds of 256 whole tiles write C directly, the tiles left
@@ -216,7 +216,7 @@ def test_tile_k_slices_for_the_last_partial_round(pkg, oracle, variant, split, s
     assert np.isfinite(C).all()
 
 
-@pytest.mark.parametrize("variant", [None, 0, 1, 5, 6])
+@pytest.mark.parametrize("variant", [None, 0, 5, 6])
 @pytest.mark.parametrize("shape", [(256, 16, 256), (300, 1000 // 16 * 16 + 16, 200), (512, 2000, 520), (1100, 4112, 700),
                                    (64, 1040, 512), (16, 8176, 1024)])
 def test_k_that_is_only_a_multiple_of_16(pkg, oracle, variant, shape):
@@ -236,12 +236,12 @@ def test_k_that_is_only_a_multiple_of_16(pkg, oracle, variant, shape):
     assert worst < 0.5
 
 
-@pytest.mark.parametrize("variant", [1, 7, None])
+@pytest.mark.parametrize("variant", [0, 6, None])
 @pytest.mark.parametrize("shape", [(256, 64, 256), (300, 192, 200), (1100, 448, 2100), (2048, 8256, 2304)])
 def test_odd_count_of_64_byte_k_tiles(pkg, oracle, variant, shape):
     """k % 64 == 0 but k % 128 != 0 (the reference's own requirement is k % 64 == 0,
-    GEMM/src/gemm.cu:45-47): the tiled kernels with 64-byte K tiles take it, whether picked
-    by hand or by the automatic selection."""
+    GEMM/src/gemm.cu:45-47): the last 128-byte K tile is half empty, whether the kernel is
+    picked by hand or by the automatic selection."""
     M, K, N = shape
     assert pkg.lib().fp8gemm_select_algo(M, K, N) == ALGOS["tile"]
     A = pkg.fill((M, K), 0, seed=0xA11CE + K, dist="normal", sigma=4.0)
@@ -283,7 +283,7 @@ def test_decode_through_mfma_is_bit_exact(pkg, oracle, fa, fb, algo):
     exactly, for every finite code, and likewise with the roles swapped."""
     one = {0: 0x38, 1: 0x3C}
     K = 256
-    M = 64 if algo == "skinny" else 256
+    M = 16 if algo == "skinny" else 256
     N = 256
     rng = np.random.default_rng(7)
     ks = rng.permutation(K)[:M] if M <= K else rng.integers(0, K, M)
@@ -309,12 +309,12 @@ def test_decode_through_mfma_is_bit_exact(pkg, oracle, fa, fb, algo):
     assert np.array_equal(C2, oracle.decode(A2, fa)[:, kn])
 
 
-@pytest.mark.parametrize("algo,variant", [("tile", 13), ("tile", 14), ("tile", 5), ("tile", 6), ("tile", 8), ("tile", 1), ("tile", 15),
+@pytest.mark.parametrize("algo,variant", [("tile", 13), ("tile", 14), ("tile", 5), ("tile", 6), ("tile", 8), ("tile", 9), ("tile", 15),
                                           ("tile", 16)])
 @pytest.mark.parametrize("fa,fb", PAIRS)
 def test_decode_through_mfma_every_persistent_form(pkg, oracle, fa, fb, algo, variant):
     """The same bit-exact selection test for the persistent tile shapes the planner uses
-    (both MFMA shapes, 2-, 3- and 4-deep rings): one-hot A selects codes of B and one-hot B
+    (both MFMA shapes, rings 2 to 5 slots deep): one-hot A selects codes of B and one-hot B
     selects codes of A, K = 512 so that the 16x16x128 forms see four K tiles."""
     one = {0: 0x38, 1: 0x3C}
     M, K, N = 384, 512, 512
@@ -350,7 +350,7 @@ def test_tall_general_kernel_shape_beyond_65535_row_tiles(pkg, oracle):
     assert np.array_equal(C, Af @ Bf.T)
 
 
-@pytest.mark.parametrize("algo,shape", [("direct", (96, 200, 64)), ("tile", (256, 1024, 256)), ("skinny", (48, 1024, 128))])
+@pytest.mark.parametrize("algo,shape", [("direct", (96, 200, 64)), ("tile", (256, 1024, 256)), ("skinny", (12, 1024, 128))])
 def test_small_integers_are_exact(pkg, oracle, algo, shape):
     """|values| <= 8 and K <= 2^10: every partial sum is an integer below 2^24, so any
     summation order gives the same bits as the oracle."""
@@ -469,17 +469,18 @@ def test_caller_provided_workspace(pkg, oracle):
     import torch
     L = pkg.lib()
     stream = torch.cuda.current_stream().cuda_stream
-    for (M, K, N) in [(256, 8192, 2048), (64, 8192, 2048), (512, 1024, 768)]:
+    for (M, K, N), stages in [((256, 8192, 2048), 2), ((64, 8192, 2048), 2), ((512, 1024, 768), 2),
+                              ((256, 28672, 10240), 4), ((256, 4912, 6144), 4)]:
         need = L.fp8gemm_scratch_bytes(M, K, N)
         A = pkg.fill((M, K), 0, seed=0xA11CE + 500 + M, dist="normal", sigma=2.0)
         B = pkg.fill((N, K), 0, seed=0xB0B + 500 + M, dist="normal", sigma=2.0)
         dA, dB = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
         ref = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
-        pkg.gemm(dA, dB, out=ref, a_fmt=0, b_fmt=0)
+        pkg.gemm(dA, dB, out=ref, a_fmt=0, b_fmt=0, stages=stages)
         got = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
         ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
         held = L.fp8gemm_scratch_held_bytes()
-        code = L.fp8gemm_launch_ws(M, K, N, dA.data_ptr(), 0, dB.data_ptr(), 0, got.data_ptr(), 2,
+        code = L.fp8gemm_launch_ws(M, K, N, dA.data_ptr(), 0, dB.data_ptr(), 0, got.data_ptr(), stages,
                                    ws.data_ptr() if need else None, need, stream)
         assert code == 0
         torch.cuda.synchronize()
@@ -488,11 +489,11 @@ def test_caller_provided_workspace(pkg, oracle):
         assert_within_bound(oracle, got.cpu().numpy(), A, 0, B, 0)
         if need:
             got.fill_(float("nan"))
-            assert L.fp8gemm_launch_ws(M, K, N, dA.data_ptr(), 0, dB.data_ptr(), 0, got.data_ptr(), 2,
+            assert L.fp8gemm_launch_ws(M, K, N, dA.data_ptr(), 0, dB.data_ptr(), 0, got.data_ptr(), stages,
                                        ws.data_ptr(), need - 1, stream) == 2
-            assert L.fp8gemm_launch_ws(M, K, N, dA.data_ptr(), 0, dB.data_ptr(), 0, got.data_ptr(), 2,
+            assert L.fp8gemm_launch_ws(M, K, N, dA.data_ptr(), 0, dB.data_ptr(), 0, got.data_ptr(), stages,
                                        None, 0, stream) == 2
-            assert L.fp8gemm_launch_ws(M, K, N, dA.data_ptr(), 0, dB.data_ptr(), 0, got.data_ptr(), 2,
+            assert L.fp8gemm_launch_ws(M, K, N, dA.data_ptr(), 0, dB.data_ptr(), 0, got.data_ptr(), stages,
                                        ws.data_ptr() + 4, need, stream) == 1      # misaligned workspace
             torch.cuda.synchronize()
             assert bool(torch.isnan(got).all())             # nothing was launched
