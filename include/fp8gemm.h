@@ -74,6 +74,52 @@ int fp8gemm_launch(int m, int k, int n, const void *a, int a_fmt, const void *b,
 int fp8gemm_gemv(int n, int k, const void *w, int w_fmt, const void *x, int x_fmt, float *y, void *stream);
 
 /*
+ * ---- Sparse operands: SpMM and SpMV ---------------------------------------------------
+ * out = S * B^T with S (m x k) sparse and B dense, stored n x k like the B of the GEMM; out is
+ * m x n fp32 row-major, overwritten; n = 1 with a vector x of k codes is the SpMV.  The
+ * reference names SpMM and SpMV as planned kernels (README.md:7) and holds none; what it holds
+ * are the host helpers that generate the two operand formats taken here
+ * (GEMM/include/bm_test_utils.h:48-68 blocked-ELL column lists, :71-128 compressed sparse rows
+ * with optional row padding, :197-216 row orders).  Every stored entry contributes
+ * float(value) * float(b[j][column]) to out[i][j], fp32 accumulation; all pointers are device
+ * pointers; formats as for the GEMM; launches are asynchronous on `stream`.
+ *
+ * Blocked-ELL: square blocks of `block` x `block` elements (block % 16 == 0, m % block == 0,
+ * k % block == 0); every block row stores ell_cols blocks.  values: m x (ell_cols * block)
+ * codes row-major, 16-byte aligned (stored block t of a row's block row occupies bytes
+ * t * block .. of the row); block_cols: (m / block) x ell_cols ints, the block column of each
+ * stored block, or -1 for a padding block that contributes nothing.  The kernel feeds the MFMA
+ * from the stored blocks directly; blocks that are not stored cost nothing.  b 16-byte aligned.
+ */
+int fp8gemm_spmm_bell(int m, int k, int n, int block, int ell_cols, const void *values, int s_fmt, const int *block_cols,
+                      const void *b, int b_fmt, float *out, void *stream);
+int fp8gemm_spmv_bell(int m, int k, int block, int ell_cols, const void *values, int s_fmt, const int *block_cols,
+                      const void *x, int x_fmt, float *y, void *stream);
+/*
+ * Compressed sparse rows: values (codes), row_offsets (m + 1 ints, ascending from 0), col_idx
+ * (ints in [0, k)).  fp8gemm_spmv_csr streams values and indices once, one wave per row, rows
+ * taken in the order row_order gives (m ints, a permutation of 0 .. m-1, e.g. longest rows
+ * first, see fp8gemm_sorted_row_swizzle; NULL = 0, 1, 2, ..); entries of a row that name the same
+ * column are added.  fp8gemm_spmm_csr writes S out as a dense m x k fp8 matrix in the stream's
+ * scratch (fp8gemm_spmm_csr_scratch_bytes tells how much it takes from the per-stream pool
+ * described under "Device scratch") and runs the dense GEMM on it: no matrix instruction takes
+ * single elements, and with B stored n x k an element-wise kernel would gather single bytes.
+ * For this one the columns of a row must be distinct, except that entries whose value is +-0
+ * may repeat a column (the zero padding of the reference's generator does) and are skipped.
+ */
+int fp8gemm_spmv_csr(int m, int k, const void *values, int s_fmt, const int *row_offsets, const int *col_idx,
+                     const int *row_order, const void *x, int x_fmt, float *y, void *stream);
+int fp8gemm_spmm_csr(int m, int k, int n, const void *values, int s_fmt, const int *row_offsets, const int *col_idx,
+                     const void *b, int b_fmt, float *out, void *stream);
+size_t fp8gemm_spmm_csr_scratch_bytes(int m, int k, int n);
+/*
+ * Host helper: rows ordered by falling number of stored entries (ties in rising row number),
+ * the order of the reference's SortedRowSwizzle (GEMM/include/bm_test_utils.h:202-216).
+ * row_offsets and row_indices are HOST arrays of m + 1 and m ints.
+ */
+void fp8gemm_sorted_row_swizzle(int m, const int *row_offsets, int *row_indices);
+
+/*
  * Extended epilogue, with no counterpart in the reference's gemm:: API; it covers what the
  * reference's vendor-library sample hands to cuBLASLt next to the operands
  * (GEMM/src/cublas.cu:9-23, 41-46; GEMM/include/helper.h:84, 125, 159-160: host alpha and

@@ -5,7 +5,9 @@ cpu_baseline leg of bench.py as the checker.  The library and its harness never
 import it.
 
 The reference path it restates: GEMM/gemm_main.cpp:39-53 (fp32 CPU GEMM over
-fp8 inputs) with the fp8 types of GEMM/include/gemm.cuh:6-7.
+fp8 inputs) with the fp8 types of GEMM/include/gemm.cuh:6-7; the sparse-times-dense
+loop is that loop over the stored entries of the reference's sparse operand formats
+(GEMM/include/bm_test_utils.h:48-128), for which the reference holds no loop of its own.
 """
 import ctypes
 import os
@@ -52,6 +54,8 @@ def lib():
     L.oracle_gemm_fast.restype = None
     L.oracle_gemm_fast.argtypes = [ctypes.c_int] * 3 + [u8p, ctypes.c_int, u8p, ctypes.c_int,
                                                         i32p, ctypes.c_int, f32p, f64p]
+    L.oracle_spmm_csr.restype = None
+    L.oracle_spmm_csr.argtypes = [ctypes.c_int] * 3 + [u8p, ctypes.c_int, i32p, i32p, u8p, ctypes.c_int, f32p, f64p]
     L.oracle_num_threads.restype = ctypes.c_int
     L.oracle_set_num_threads.argtypes = [ctypes.c_int]
     _lib = L
@@ -112,6 +116,48 @@ def gemm(A, afmt, B, bfmt, rows=None, with_scale=False):
     lib().oracle_gemm_fast(M, K, N, _p(A, ctypes.c_uint8), afmt, _p(B, ctypes.c_uint8), bfmt,
                            rp, R, _p(C, ctypes.c_float), _p(S, ctypes.c_double) if with_scale else None)
     return (C, S) if with_scale else C
+
+
+def spmm_csr(values, sfmt, row_offsets, col, k, B, bfmt, with_scale=False):
+    """Sparse (CSR, m x k) times dense (B stored n x k) -> m x n fp32, entries of a row added in
+    storage order as a running fp32 sum.  A one-dimensional B (k codes) is the SpMV and gives m floats."""
+    values = np.ascontiguousarray(values, dtype=np.uint8)
+    row_offsets = np.ascontiguousarray(row_offsets, dtype=np.int32)
+    col = np.ascontiguousarray(col, dtype=np.int32)
+    B = np.ascontiguousarray(B, dtype=np.uint8)
+    vector = B.ndim == 1
+    B2 = B.reshape(1, -1) if vector else B
+    m, (n, k2) = row_offsets.size - 1, B2.shape
+    assert k == k2 and row_offsets[0] == 0 and row_offsets[-1] == values.size == col.size
+    assert col.size == 0 or (col.min() >= 0 and col.max() < k)
+    out = np.empty((m, n), dtype=np.float32)
+    S = np.empty((m, n), dtype=np.float64) if with_scale else None
+    lib().oracle_spmm_csr(m, k, n, _p(values, ctypes.c_uint8), sfmt, _p(row_offsets, ctypes.c_int), _p(col, ctypes.c_int),
+                          _p(B2, ctypes.c_uint8), bfmt, _p(out, ctypes.c_float), _p(S, ctypes.c_double) if with_scale else None)
+    if vector:
+        out = out[:, 0]
+        S = S[:, 0] if with_scale else None
+    return (out, S) if with_scale else out
+
+
+def bell_to_csr(values, block_cols, block):
+    """Blocked-ELL (the format behind the reference's GenerateUniformBlockedELLIndex,
+    GEMM/include/bm_test_utils.h:48-68: square blocks of `block`, every block row stores the same
+    number of blocks; values m x (ell_cols*block) codes, block_cols (m/block) x ell_cols block
+    column numbers, -1 = padding that holds nothing) -> (values, row_offsets, col) in CSR, every
+    stored element of a block an entry (zeros included), in storage order."""
+    values = np.ascontiguousarray(values, dtype=np.uint8)
+    block_cols = np.ascontiguousarray(block_cols, dtype=np.int32)
+    m, kell = values.shape
+    nbr, ell = block_cols.shape
+    assert m == nbr * block and kell == ell * block
+    cols = (block_cols[:, :, None] * block + np.arange(block, dtype=np.int32)[None, None, :]).reshape(nbr, kell)
+    keep = np.repeat(block_cols >= 0, block, axis=1)                    # (nbr, kell)
+    keep_rows = np.repeat(keep, block, axis=0)                          # (m, kell)
+    cols_rows = np.repeat(cols, block, axis=0)
+    row_offsets = np.zeros(m + 1, dtype=np.int32)
+    row_offsets[1:] = np.cumsum(keep_rows.sum(axis=1))
+    return values[keep_rows], row_offsets, cols_rows[keep_rows].astype(np.int32)
 
 
 def tolerance(K, S):

@@ -115,6 +115,19 @@ def lib():
     L.fp8gemm_fill_weights.argtypes = [vp, ctypes.c_size_t, ci, ctypes.c_uint64, ctypes.c_float]
     L.fp8gemm_fill_loguniform.restype = None
     L.fp8gemm_fill_loguniform.argtypes = [vp, ctypes.c_size_t, ci, ctypes.c_uint64]
+    ip = ctypes.c_void_p
+    L.fp8gemm_spmm_bell.restype = ci
+    L.fp8gemm_spmm_bell.argtypes = [ci, ci, ci, ci, ci, vp, ci, ip, vp, ci, vp, vp]
+    L.fp8gemm_spmv_bell.restype = ci
+    L.fp8gemm_spmv_bell.argtypes = [ci, ci, ci, ci, vp, ci, ip, vp, ci, vp, vp]
+    L.fp8gemm_spmv_csr.restype = ci
+    L.fp8gemm_spmv_csr.argtypes = [ci, ci, vp, ci, ip, ip, ip, vp, ci, vp, vp]
+    L.fp8gemm_spmm_csr.restype = ci
+    L.fp8gemm_spmm_csr.argtypes = [ci, ci, ci, vp, ci, ip, ip, vp, ci, vp, vp]
+    L.fp8gemm_spmm_csr_scratch_bytes.restype = ctypes.c_size_t
+    L.fp8gemm_spmm_csr_scratch_bytes.argtypes = [ci, ci, ci]
+    L.fp8gemm_sorted_row_swizzle.restype = None
+    L.fp8gemm_sorted_row_swizzle.argtypes = [ci, ip, ip]
     _lib = L
     return L
 
@@ -292,3 +305,72 @@ def GEMM(m, k, n, a, b, out):
 def GEMM4(m, k, n, a, b, out):
     """gemm::GEMM4 of the reference (gemm.cuh:18-21, 30-33, 41-44, 52-55)."""
     return _entry(m, k, n, a, b, out, 4)
+
+
+# ---------------------------------------------------------------- sparse operands
+def _dev_ints(t):
+    import torch
+    if not (t.is_cuda and t.dtype == torch.int32 and t.is_contiguous()):
+        raise Fp8GemmError("index arrays are contiguous int32 device tensors")
+    return t.data_ptr()
+
+
+def spmm_bell(values, block_cols, block, b, k, s_fmt=None, b_fmt=None, out=None, stream=None):
+    """out[m, n] = S b^T for S (m x k) in blocked-ELL: values (m, ell_cols*block) codes, block_cols
+    (m/block, ell_cols) int32 block column numbers (-1 = padding), b (n, k) dense; device tensors.
+    A one-dimensional b (k codes) is the matrix-vector product and gives m floats."""
+    import torch
+    m, kell = values.shape
+    ell_cols = block_cols.shape[1]
+    if kell != ell_cols * block or block_cols.shape[0] * block != m:
+        raise Fp8GemmError("values / block_cols do not fit the block size")
+    vector = b.dim() == 1
+    n = 1 if vector else b.shape[0]
+    if (b.shape[0] if vector else b.shape[1]) != k:
+        raise Fp8GemmError("b does not have k columns")
+    if out is None:
+        out = torch.empty((m,) if vector else (m, n), dtype=torch.float32, device=values.device)
+    L = lib()
+    fs, fb = _fmt_of(values, s_fmt), _fmt_of(b, b_fmt)
+    if vector:
+        code = L.fp8gemm_spmv_bell(m, k, block, ell_cols, values.data_ptr(), fs, _dev_ints(block_cols), b.data_ptr(), fb,
+                                   out.data_ptr(), _stream_handle(stream))
+    else:
+        code = L.fp8gemm_spmm_bell(m, k, n, block, ell_cols, values.data_ptr(), fs, _dev_ints(block_cols), b.data_ptr(), fb,
+                                   out.data_ptr(), _stream_handle(stream))
+    check(code)
+    return out
+
+
+def spmm_csr(values, row_offsets, col_idx, b, k, s_fmt=None, b_fmt=None, out=None, row_order=None, stream=None):
+    """out = S b^T for S (m x k) in compressed sparse rows (values codes, row_offsets m+1 and col_idx
+    int32; device tensors), b (n, k) dense, or a vector of k codes for the matrix-vector product
+    (row_order: optional int32 permutation of the rows, the order the waves take them in)."""
+    import torch
+    m = row_offsets.numel() - 1
+    vector = b.dim() == 1
+    n = 1 if vector else b.shape[0]
+    if (b.shape[0] if vector else b.shape[1]) != k:
+        raise Fp8GemmError("b does not have k columns")
+    if out is None:
+        out = torch.empty((m,) if vector else (m, n), dtype=torch.float32, device=values.device)
+    L = lib()
+    fs, fb = _fmt_of(values, s_fmt), _fmt_of(b, b_fmt)
+    if vector:
+        code = L.fp8gemm_spmv_csr(m, k, values.data_ptr(), fs, _dev_ints(row_offsets), _dev_ints(col_idx),
+                                  None if row_order is None else _dev_ints(row_order), b.data_ptr(), fb, out.data_ptr(),
+                                  _stream_handle(stream))
+    else:
+        code = L.fp8gemm_spmm_csr(m, k, n, values.data_ptr(), fs, _dev_ints(row_offsets), _dev_ints(col_idx), b.data_ptr(), fb,
+                                  out.data_ptr(), _stream_handle(stream))
+    check(code)
+    return out
+
+
+def sorted_row_swizzle(row_offsets):
+    """Host: rows ordered by falling number of stored entries (numpy int32 in, numpy int32 out)."""
+    import numpy as np
+    row_offsets = np.ascontiguousarray(row_offsets, dtype=np.int32)
+    out = np.empty(row_offsets.size - 1, dtype=np.int32)
+    lib().fp8gemm_sorted_row_swizzle(out.size, row_offsets.ctypes.data, out.ctypes.data)
+    return out

@@ -113,9 +113,11 @@ hipError_t launch_ptile_shape_k(int m, int k, int n, const uint8_t *a, const uin
     // Scratch of a K-sliced launch: arrival counters, then the partial sums.  For tiles up to
     // 128 x 128, where the counters can be relied on (see Workspace), the slice of a tile that
     // arrives last adds the slices up inside the kernel; otherwise a reduction kernel follows.
-    // (One CU adding up four slices of a 256 x 256 tile reads 1 MiB: measured 6 to 15 us slower
-    // than the reduction kernel, which spreads that over the chip; for a 64 x 128 tile it is 128 KiB
-    // and 1 to 2 us faster than a second launch.)
+    // (One CU adding up the slices of a larger tile is slower than the reduction kernel, which
+    // spreads that over the chip.  MI355X, M=256, weights cold, sum in the kernel / by the reduction
+    // kernel: 128 x 256 tiles in 3 slices at N=10240 K=8192 41.3 / 38.2 us, 256 x 128 in 4 slices at
+    // N=8192 K=28672 75.1 / 69.8 us, 256 x 256 in 2 slices at N=28672 K=8192 76.2 / 73.0 us;
+    // for a 64 x 128 tile it is 128 KiB per tile and 1 to 2 us faster than a second launch.)
     constexpr bool kSumInKernel = ptile_sums_slices_in_kernel<S>;
     float *base = nullptr, *ws = nullptr;
     int *counters = nullptr;

@@ -14,6 +14,7 @@
 #include <utility>
 
 #include "kernel_reduce.h"
+#include "kernel_sparse.h"
 #include "plan.h"
 #include "scratch_pool.h"
 
@@ -427,6 +428,43 @@ int launch_pooled(int m, int k, int n, const void *a, int a_fmt, const void *b, 
 
 using namespace fp8gemm_detail;
 
+// ------------------------------------------------------------------ sparse operands
+namespace {
+
+template <int SF, int BF>
+hipError_t launch_spmm_bell(int m, int k, int n, int block, int ell_cols, const uint8_t *values, const int *block_cols,
+                            const uint8_t *b, float *out, hipStream_t stream)
+{
+    // columns of out per wave: as many as n fills, up to 64
+    const int tn = n <= 16 ? 1 : (n <= 32 ? 2 : 4);
+    const long groups_n = (n + 16 * tn - 1) / (16 * tn);
+    const long grid = (long)(m / 16) * groups_n;
+    if (grid > 0x7FFFFFFFL) return hipErrorInvalidValue;
+    if (tn == 1)
+        hipLaunchKernelGGL((spmm_bell_kernel<SF, BF, 1>), dim3((unsigned)grid), dim3(64), 0, stream, m, k, n, block, ell_cols,
+                           values, block_cols, b, out, (int)groups_n);
+    else if (tn == 2)
+        hipLaunchKernelGGL((spmm_bell_kernel<SF, BF, 2>), dim3((unsigned)grid), dim3(64), 0, stream, m, k, n, block, ell_cols,
+                           values, block_cols, b, out, (int)groups_n);
+    else
+        hipLaunchKernelGGL((spmm_bell_kernel<SF, BF, 4>), dim3((unsigned)grid), dim3(64), 0, stream, m, k, n, block, ell_cols,
+                           values, block_cols, b, out, (int)groups_n);
+    return hipGetLastError();
+}
+
+template <int SF, int XF>
+hipError_t launch_spmv_csr(int m, const uint8_t *values, const int *row_offsets, const int *col, const int *row_order,
+                           const uint8_t *x, float *y, hipStream_t stream)
+{
+    hipLaunchKernelGGL((spmv_csr_kernel<SF, XF>), dim3((unsigned)((m + 3) / 4)), dim3(256), 0, stream, m, values, row_offsets,
+                       col, row_order, x, y);
+    return hipGetLastError();
+}
+
+bool fmt_ok(int f) { return f == FP8GEMM_E4M3 || f == FP8GEMM_E5M2; }
+
+}  // namespace
+
 extern "C" {
 
 int fp8gemm_launch(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,
@@ -438,6 +476,91 @@ int fp8gemm_launch(int m, int k, int n, const void *a, int a_fmt, const void *b,
 int fp8gemm_gemv(int n, int k, const void *w, int w_fmt, const void *x, int x_fmt, float *y, void *stream)
 {
     return launch_pooled(1, k, n, x, x_fmt, w, w_fmt, y, 2, FP8GEMM_ALGO_AUTO, -1, 0, stream);
+}
+
+// ------------------------------------------------------------------ sparse operands
+int fp8gemm_spmm_bell(int m, int k, int n, int block, int ell_cols, const void *values, int s_fmt, const int *block_cols,
+                      const void *b, int b_fmt, float *out, void *stream)
+{
+    if (m <= 0 || k <= 0 || n <= 0 || block <= 0 || ell_cols <= 0 || !values || !block_cols || !b || !out)
+        return (int)hipErrorInvalidValue;
+    if (!fmt_ok(s_fmt) || !fmt_ok(b_fmt)) return (int)hipErrorInvalidValue;
+    if (block % 16 != 0 || m % block != 0 || k % block != 0) return (int)hipErrorInvalidValue;
+    if ((long)ell_cols * block > (1L << 30)) return (int)hipErrorInvalidValue;
+    if ((reinterpret_cast<uintptr_t>(values) | reinterpret_cast<uintptr_t>(b)) % 16 != 0) return (int)hipErrorInvalidValue;
+    const uint8_t *pv = static_cast<const uint8_t *>(values), *pb = static_cast<const uint8_t *>(b);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    (void)hipGetLastError();
+    hipError_t e;
+    if (s_fmt == FP8GEMM_E4M3 && b_fmt == FP8GEMM_E4M3)
+        e = launch_spmm_bell<0, 0>(m, k, n, block, ell_cols, pv, block_cols, pb, out, s);
+    else if (s_fmt == FP8GEMM_E5M2 && b_fmt == FP8GEMM_E5M2)
+        e = launch_spmm_bell<1, 1>(m, k, n, block, ell_cols, pv, block_cols, pb, out, s);
+    else if (s_fmt == FP8GEMM_E4M3)
+        e = launch_spmm_bell<0, 1>(m, k, n, block, ell_cols, pv, block_cols, pb, out, s);
+    else
+        e = launch_spmm_bell<1, 0>(m, k, n, block, ell_cols, pv, block_cols, pb, out, s);
+    return (int)e;
+}
+
+int fp8gemm_spmv_bell(int m, int k, int block, int ell_cols, const void *values, int s_fmt, const int *block_cols,
+                      const void *x, int x_fmt, float *y, void *stream)
+{
+    return fp8gemm_spmm_bell(m, k, 1, block, ell_cols, values, s_fmt, block_cols, x, x_fmt, y, stream);
+}
+
+int fp8gemm_spmv_csr(int m, int k, const void *values, int s_fmt, const int *row_offsets, const int *col_idx,
+                     const int *row_order, const void *x, int x_fmt, float *y, void *stream)
+{
+    if (m <= 0 || k <= 0 || !values || !row_offsets || !col_idx || !x || !y) return (int)hipErrorInvalidValue;
+    if (!fmt_ok(s_fmt) || !fmt_ok(x_fmt)) return (int)hipErrorInvalidValue;
+    const uint8_t *pv = static_cast<const uint8_t *>(values), *px = static_cast<const uint8_t *>(x);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    (void)hipGetLastError();
+    hipError_t e;
+    if (s_fmt == FP8GEMM_E4M3 && x_fmt == FP8GEMM_E4M3)
+        e = launch_spmv_csr<0, 0>(m, pv, row_offsets, col_idx, row_order, px, y, s);
+    else if (s_fmt == FP8GEMM_E5M2 && x_fmt == FP8GEMM_E5M2)
+        e = launch_spmv_csr<1, 1>(m, pv, row_offsets, col_idx, row_order, px, y, s);
+    else if (s_fmt == FP8GEMM_E4M3)
+        e = launch_spmv_csr<0, 1>(m, pv, row_offsets, col_idx, row_order, px, y, s);
+    else
+        e = launch_spmv_csr<1, 0>(m, pv, row_offsets, col_idx, row_order, px, y, s);
+    return (int)e;
+}
+
+size_t fp8gemm_spmm_csr_scratch_bytes(int m, int k, int n)
+{
+    if (m <= 0 || k <= 0 || n <= 0) return 0;
+    const size_t dense = ((size_t)m * k + 255) / 256 * 256;
+    return kSliceCounterBytes + dense + fp8gemm_scratch_bytes(m, k, n);
+}
+
+int fp8gemm_spmm_csr(int m, int k, int n, const void *values, int s_fmt, const int *row_offsets, const int *col_idx,
+                     const void *b, int b_fmt, float *out, void *stream)
+{
+    if (m <= 0 || k <= 0 || n <= 0 || !values || !row_offsets || !col_idx || !b || !out) return (int)hipErrorInvalidValue;
+    if (!fmt_ok(s_fmt) || !fmt_ok(b_fmt)) return (int)hipErrorInvalidValue;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // scratch of this stream: [arrival counters of the pool's buffer, left alone | S as a dense m x k
+    // fp8 matrix | the workspace of the dense GEMM]
+    const size_t dense_bytes = ((size_t)m * k + 255) / 256 * 256;
+    const size_t gemm_bytes = fp8gemm_scratch_bytes(m, k, n);
+    Workspace pool = Workspace::pooled(s);
+    void *p = nullptr;
+    hipError_t e = pool.get(kSliceCounterBytes + dense_bytes + gemm_bytes, &p);
+    if (e != hipSuccess) return (int)e;
+    uint8_t *dense = static_cast<uint8_t *>(p) + kSliceCounterBytes;
+    (void)hipGetLastError();
+    const size_t count16 = dense_bytes / 16;
+    hipLaunchKernelGGL(zero_bytes16_kernel, dim3((unsigned)((count16 + 255) / 256)), dim3(256), 0, s,
+                       reinterpret_cast<v4i *>(dense), count16);
+    hipLaunchKernelGGL(csr_densify_kernel, dim3((unsigned)((m + 3) / 4)), dim3(256), 0, s, m, (size_t)k,
+                       static_cast<const uint8_t *>(values), row_offsets, col_idx, dense);
+    e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    Workspace gemm_ws = Workspace::fixed(gemm_bytes ? dense + dense_bytes : nullptr, gemm_bytes, false);
+    return launch_checked(m, k, n, dense, s_fmt, b, b_fmt, out, 2, FP8GEMM_ALGO_AUTO, -1, 0, stream, kPlainOut, gemm_ws);
 }
 
 int fp8gemm_launch_ws(int m, int k, int n, const void *a, int a_fmt, const void *b, int b_fmt,

@@ -1,10 +1,12 @@
 // Host-side helpers exported through the C ABI: the bit-exact fp8 codec in bulk
-// form and the seeded synthetic matrix generators.  They play the role of the
+// form, the seeded synthetic matrix generators and the row order of the sparse kernels.  They play the role of the
 // fp8 converting constructors and MakeDenseMatrix in the reference's harness
 // (GEMM/include/bm_test_utils.h:131-143) with explicit seeds and distributions.
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
 #include <cstring>
+#include <numeric>
 
 #include "fp8.h"
 #include "fp8gemm.h"
@@ -48,6 +50,14 @@ void fp8gemm_fill_weights(uint8_t *dst, size_t count, int fmt, uint64_t seed, fl
 void fp8gemm_fill_loguniform(uint8_t *dst, size_t count, int fmt, uint64_t seed)
 {
     synth::fill_loguniform(dst, count, fmt, seed);
+}
+
+void fp8gemm_sorted_row_swizzle(int m, const int *row_offsets, int *row_indices)
+{
+    std::iota(row_indices, row_indices + m, 0);
+    std::stable_sort(row_indices, row_indices + m, [row_offsets](int a, int b) {
+        return row_offsets[a + 1] - row_offsets[a] > row_offsets[b + 1] - row_offsets[b];
+    });
 }
 
 }  // extern "C"

@@ -1,0 +1,181 @@
+"""GPU parity of the sparse-times-dense entry points (blocked-ELL and CSR, SpMM and SpMV),
+called through the C ABI, against the CPU oracle's sparse loop (oracle_spmm_csr, which
+tests/test_oracle_sparse.py pins without the reference: the reference holds no SpMM / SpMV
+kernel, loop or vector, only the generators of the operand formats,
+GEMM/include/bm_test_utils.h:48-128).
+
+Bar: |out_gpu - out_ref| <= 2 * L * 2^-24 * sum |a*b| per element, L = stored entries of the
+row (reordered fp32 accumulation only; products are exact), plus the MFMA's alignment-window
+term where the sums are short; bit-exact where no rounding can occur.
+"""
+import zlib
+
+import numpy as np
+import pytest
+
+from conftest import finite_codes, random_codes
+from sparse_util import random_bell, random_csr
+
+pytestmark = pytest.mark.gpu
+
+PAIRS = [(0, 0), (1, 1), (0, 1), (1, 0)]
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def bound(oracle, vals, sfmt, offs, col, k, B, bfmt, mfma=False):
+    """Reference, and the tolerance per element."""
+    ref, S = oracle.spmm_csr(vals, sfmt, offs, col, k, B, bfmt, with_scale=True)
+    L = np.diff(offs).astype(np.float64)
+    L = L if S.ndim == 1 else L[:, None]
+    tol = 2.0 * np.maximum(L, 1.0) * 2.0 ** -24 * S
+    if mfma:
+        # the f8f6f4 MFMA adds groups of 8 products with 13 bits below the group's largest
+        # (tests/test_gpu_mfma_numerics.py); bounded here by 2^-10 of the largest product times the group count
+        amax = np.abs(oracle.decode(vals, sfmt)).max() if vals.size else 0.0
+        bmax = np.abs(oracle.decode(B, bfmt)).max()
+        tol = tol + 2.0 ** -10 * amax * bmax * np.maximum(L, 1.0) / 8.0
+    return ref, tol
+
+
+def check(out, ref, tol):
+    assert np.isfinite(out).all()
+    err = np.abs(out.astype(np.float64) - ref.astype(np.float64))
+    assert (err <= tol).all(), "worst err/tol = %g" % float((err / np.maximum(tol, 1e-300)).max())
+
+
+@pytest.mark.parametrize("fs,fb", PAIRS)
+@pytest.mark.parametrize("block,ell,m,k,n", [(16, 3, 64, 160, 40), (32, 5, 128, 512, 100), (64, 2, 256, 1024, 64),
+                                              (128, 3, 256, 2048, 33), (48, 2, 96, 480, 17), (16, 9, 32, 144, 16)])
+def test_spmm_bell_all_finite_codes(pkg, oracle, fs, fb, block, ell, m, k, n):
+    """Every finite code as a value, padding blocks included, block sizes that are and are not
+    powers of two, stored rows that are not whole 128-byte K steps, n that overhangs the wave's
+    column group."""
+    rng = np.random.default_rng(zlib.crc32(repr((fs, fb, block, ell, m, k, n)).encode()))
+    vals, bcols = random_bell(rng, m, k, block, ell, fs, pad_some=True)
+    B = random_codes(rng, (n, k), fb)
+    if fb == 1:
+        B = np.where(((B >> 2) & 0x1F) > 24, B & 0x83 | 0x3C, B).astype(np.uint8)
+    out = pkg.spmm_bell(dev(vals), dev(bcols), block, dev(B), k, s_fmt=fs, b_fmt=fb).cpu().numpy()
+    v, offs, col = oracle.bell_to_csr(vals, bcols, block)
+    ref, tol = bound(oracle, v, fs, offs, col, k, B, fb, mfma=True)
+    check(out, ref, tol)
+
+
+@pytest.mark.parametrize("fs,fb", PAIRS)
+def test_spmm_bell_normal_values_plain_bound(pkg, oracle, fs, fb):
+    """N(0,1)-like values, long stored rows: the plain reordering bound, no hardware term."""
+    rng = np.random.default_rng(31 + fs * 2 + fb)
+    m, k, n, block, ell = 512, 8192, 256, 64, 32
+    vals, bcols = random_bell(rng, m, k, block, ell, fs, encode=oracle.encode, sigma=2.0)
+    B = pkg.fill((n, k), fb, seed=0xB0B + 70 + fs, dist="normal", sigma=2.0)
+    out = pkg.spmm_bell(dev(vals), dev(bcols), block, dev(B), k, s_fmt=fs, b_fmt=fb).cpu().numpy()
+    v, offs, col = oracle.bell_to_csr(vals, bcols, block)
+    ref, tol = bound(oracle, v, fs, offs, col, k, B, fb)
+    check(out, ref, tol)
+
+
+@pytest.mark.parametrize("fs,fb", PAIRS)
+def test_spmm_bell_one_hot_is_bit_exact(pkg, oracle, fs, fb):
+    """One value of 1.0 per row of S: out[i][j] == decode(b[j][that column]) for every finite
+    code of b's format (decode through the MFMA, positions gathered through the block list)."""
+    one = {0: 0x38, 1: 0x3C}
+    block, ell, m, k, n = 16, 4, 64, 256, 256
+    rng = np.random.default_rng(77 + fs)
+    _, bcols = random_bell(rng, m, k, block, ell, fs)
+    vals = np.zeros((m, ell * block), dtype=np.uint8)
+    pos = rng.integers(0, ell * block, m)
+    vals[np.arange(m), pos] = one[fs]
+    col = bcols[np.arange(m) // block, pos // block] * block + pos % block
+    codes = finite_codes(fb)
+    B = codes[rng.integers(0, codes.size, (n, k))]
+    B[:, col[0]] = np.resize(codes, n)
+    out = pkg.spmm_bell(dev(vals), dev(bcols), block, dev(B), k, s_fmt=fs, b_fmt=fb).cpu().numpy()
+    assert np.array_equal(out, oracle.decode(B, fb)[:, col].T)
+
+
+@pytest.mark.parametrize("fs,fx", PAIRS)
+@pytest.mark.parametrize("block,ell,m,k", [(16, 8, 1024, 2048), (128, 4, 512, 4096), (32, 1, 64, 64)])
+def test_spmv_bell(pkg, oracle, fs, fx, block, ell, m, k):
+    rng = np.random.default_rng(zlib.crc32(repr((fs, fx, block, ell, m, k)).encode()))
+    vals, bcols = random_bell(rng, m, k, block, ell, fs, pad_some=True, encode=oracle.encode, sigma=2.0)
+    x = pkg.fill((k,), fx, seed=0xA11CE + 80 + block, dist="normal", sigma=2.0)
+    y = pkg.spmm_bell(dev(vals), dev(bcols), block, dev(x), k, s_fmt=fs, b_fmt=fx).cpu().numpy()
+    v, offs, col = oracle.bell_to_csr(vals, bcols, block)
+    ref, tol = bound(oracle, v, fs, offs, col, k, x, fx, mfma=True)
+    check(y, ref, tol)
+
+
+@pytest.mark.parametrize("fs,fx", PAIRS)
+@pytest.mark.parametrize("m,k,density,pad", [(1000, 4096, 0.1, 0), (257, 1000, 0.3, 4), (64, 70000, 0.01, 0), (5, 7, 0.5, 0)])
+def test_spmv_csr(pkg, oracle, fs, fx, m, k, density, pad):
+    """Rows of very different lengths (empty ones included), row padding as the reference's
+    generator appends it, every finite code; natural row order and longest-rows-first."""
+    rng = np.random.default_rng(zlib.crc32(repr((fs, fx, m, k, density, pad)).encode()))
+    vals, offs, col = random_csr(rng, m, k, density, fs, all_codes=True, row_padding=pad)
+    x = random_codes(rng, (k,), fx)
+    if fx == 1:
+        x = np.where(((x >> 2) & 0x1F) > 24, x & 0x83 | 0x3C, x).astype(np.uint8)
+    ref, tol = bound(oracle, vals, fs, offs, col, k, x, fx)
+    dv, do, dc, dx = dev(vals), dev(offs), dev(col), dev(x)
+    y = pkg.spmm_csr(dv, do, dc, dx, k, s_fmt=fs, b_fmt=fx).cpu().numpy()
+    check(y, ref, tol)
+    order = pkg.sorted_row_swizzle(offs)
+    lengths = np.diff(offs)[order]
+    assert sorted(order.tolist()) == list(range(m)) and (np.diff(lengths) <= 0).all()
+    y2 = pkg.spmm_csr(dv, do, dc, dx, k, s_fmt=fs, b_fmt=fx, row_order=dev(order)).cpu().numpy()
+    assert np.array_equal(y2, y)          # the order of the rows changes no row's sum
+
+
+def test_spmv_csr_small_integers_with_duplicates_exact(pkg, oracle):
+    """|values| <= 8: every sum is an exact integer; entries that repeat a column are added."""
+    rng = np.random.default_rng(3)
+    m, k = 300, 500
+    ints = np.arange(-8, 9, dtype=np.float32)
+    counts = rng.integers(0, 200, m)
+    offs = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    col = np.concatenate([np.sort(rng.integers(0, k, c)) for c in counts]).astype(np.int32)
+    val_f = ints[rng.integers(0, ints.size, offs[-1])]
+    x_f = ints[rng.integers(0, ints.size, k)]
+    y = pkg.spmm_csr(dev(oracle.encode(val_f, 0)), dev(offs), dev(col), dev(oracle.encode(x_f, 1)), k, s_fmt=0, b_fmt=1).cpu().numpy()
+    want = np.array([np.dot(val_f[offs[i]:offs[i + 1]].astype(np.float64), x_f[col[offs[i]:offs[i + 1]]]) for i in range(m)])
+    assert np.array_equal(y.astype(np.float64), want)
+
+
+@pytest.mark.parametrize("fs,fb", PAIRS)
+@pytest.mark.parametrize("m,k,n,density,pad", [(256, 1024, 256, 0.1, 0), (300, 2048, 200, 0.05, 8), (64, 8192, 2048, 0.02, 0),
+                                                (100, 100, 50, 0.3, 0)])
+def test_spmm_csr(pkg, oracle, fs, fb, m, k, n, density, pad):
+    """Through the dense scratch and the dense GEMM (tiled kernels with and without K slices,
+    the general kernel for k % 16 != 0); zero-valued padding entries repeat a column and must
+    not wipe the real entry there."""
+    rng = np.random.default_rng(zlib.crc32(repr((fs, fb, m, k, n, density, pad)).encode()))
+    vals, offs, col = random_csr(rng, m, k, density, fs, row_padding=pad, encode=oracle.encode, sigma=2.0)
+    B = pkg.fill((n, k), fb, seed=0xB0B + 90 + m, dist="normal", sigma=2.0)
+    out = pkg.spmm_csr(dev(vals), dev(offs), dev(col), dev(B), k, s_fmt=fs, b_fmt=fb).cpu().numpy()
+    ref, S = oracle.spmm_csr(vals, fs, offs, col, k, B, fb, with_scale=True)
+    # the dense GEMM adds over all k positions (zeros included): its bound is the dense one
+    tol = oracle.tolerance(k, S) + (2.0 ** -10 * 16.0 * 16.0 if k < 1024 else 0.0)
+    check(out, ref, tol)
+    assert pkg.lib().fp8gemm_spmm_csr_scratch_bytes(m, k, n) >= m * k
+
+
+def test_sparse_entry_points_refuse_bad_arguments(pkg):
+    import torch
+    L = pkg.lib()
+    v = torch.zeros((64, 64), dtype=torch.uint8, device="cuda")
+    c = torch.zeros((4, 4), dtype=torch.int32, device="cuda")
+    b = torch.zeros((16, 64), dtype=torch.uint8, device="cuda")
+    o = torch.zeros((64, 16), dtype=torch.float32, device="cuda")
+    args = lambda block, m=64, k=64: (m, k, 16, block, 4, v.data_ptr(), 0, c.data_ptr(), b.data_ptr(), 0, o.data_ptr(), None)
+    assert L.fp8gemm_spmm_bell(*args(16)) == 0
+    assert L.fp8gemm_spmm_bell(*args(8)) == 1              # block not a multiple of 16
+    assert L.fp8gemm_spmm_bell(*args(48)) == 1             # m, k not multiples of the block
+    assert L.fp8gemm_spmm_bell(64, 64, 16, 16, 4, None, 0, c.data_ptr(), b.data_ptr(), 0, o.data_ptr(), None) == 1
+    assert L.fp8gemm_spmm_bell(64, 64, 16, 16, 4, v.data_ptr(), 2, c.data_ptr(), b.data_ptr(), 0, o.data_ptr(), None) == 1
+    assert L.fp8gemm_spmv_csr(0, 64, v.data_ptr(), 0, c.data_ptr(), c.data_ptr(), None, b.data_ptr(), 0, o.data_ptr(), None) == 1
+    assert L.fp8gemm_spmm_csr(4, 64, 16, v.data_ptr(), 0, None, c.data_ptr(), b.data_ptr(), 0, o.data_ptr(), None) == 1
+    torch.cuda.synchronize()
