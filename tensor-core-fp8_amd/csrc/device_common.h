@@ -93,6 +93,17 @@ struct OutSpec {
     float *amax;
 };
 
+// A sparse A in blocked-ELL form for the tiled kernel (kernel_sparse.h describes the format): A
+// is then the m x K matrix of stored values (K = ell_cols * block bytes per row), and K tile g of a
+// tile row pairs with the bytes of B's rows at block column cols[tile row's block row][g * BK / block].
+// block % BK == 0 and block % BM == 0, so a K tile lies inside one stored block and all rows of a
+// tile share one list.
+struct BellSpec {
+    const int *cols;      // (m / block) x ell_cols block column numbers, -1 = padding (counts as zeros)
+    int ell_cols, block;
+    int kb;               // row stride of B in bytes (the k of the sparse matrix)
+};
+
 __device__ __forceinline__ float out_scale(const OutSpec &o)
 {
     float s = o.alpha;

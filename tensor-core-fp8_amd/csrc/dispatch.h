@@ -187,6 +187,64 @@ hipError_t launch_tile(int m, int k, int n, const uint8_t *a, const uint8_t *b, 
     }
 }
 
+// ------------------------------------------------------------------ blocked-ELL A through the tiled kernel
+template <class S, int AF, int BF>
+struct PtileBellKernelTag {};
+
+template <class S, int AF, int BF>
+hipError_t launch_ptile_bell(int m, int kell, int n, const uint8_t *values, const uint8_t *b, float *out, const BellSpec &bell,
+                             int nsplit, bool split_all, int rotate, Workspace &wsp, hipStream_t stream)
+{
+    if (bell.block % S::BM != 0 || bell.block % S::BK != 0 || kell % S::BK != 0 || kell > (1 << 23) || bell.kb > (1 << 23) ||
+        nsplit < 1 || nsplit > kell / S::BK)
+        return hipErrorInvalidValue;
+    const PtileWork w = ptile_work(m, n, S::BM, S::BN, nsplit, split_all);
+    if (!w.ok) return hipErrorInvalidValue;
+    float *base = nullptr, *ws = nullptr;
+    int *counters = nullptr;
+    if (w.nsplit > 1) {
+        void *p = nullptr;
+        hipError_t e = wsp.get(ptile_scratch_bytes(w, S::BM, S::BN), &p);
+        if (e != hipSuccess) return e;
+        base = static_cast<float *>(p);
+        ws = base + kSliceCounterBytes / sizeof(float);
+        const bool window_fits = ptile_scratch_bytes(w, S::BM, S::BN) <= 0xFFFFFFFFull;
+        if (ptile_sums_slices_in_kernel<S> && wsp.counters_zero() && w.tail <= kMaxSliceCounters && window_fits)
+            counters = static_cast<int *>(p);
+    }
+    auto kernel = gemm_ptile_bell_kernel<S, AF, BF>;
+    constexpr int kLdsBytes = S::PTILE_LDS_BYTES + 256 + 16;
+    hipError_t e = allow_lds<PtileBellKernelTag<S, AF, BF>>(kernel, kLdsBytes);
+    if (e != hipSuccess) return e;
+    const int cb = tile_column_block(w.tiles_n, m, n, kell);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * w.slots)), dim3(S::THREADS), kLdsBytes, stream, m, kell, n, values, b,
+                       static_cast<void *>(out), ws, counters, w.tiles_m, w.tiles_n, w.GM, cb, w.bulk, w.tail, w.nsplit, w.rounds,
+                       rotate | (start_skew(w) << 8), bell);
+    e = hipGetLastError();
+    if (e != hipSuccess || w.nsplit == 1 || counters) return e;
+    const OutSpec plain = {1.0f, nullptr, nullptr, FP8GEMM_DEV_OUT_F32, 0.0f, nullptr, FP8GEMM_DEV_OUT_F32, nullptr, nullptr, nullptr};
+    return launch_tile_slices_reduce(base, out, m, n, kell, S::BM, S::BN, w, plain, stream);
+}
+
+template <int AF, int BF>
+hipError_t dispatch_bell(int m, int kell, int n, const uint8_t *values, const uint8_t *b, float *out, const BellSpec &bell,
+                         Workspace &wsp, hipStream_t stream)
+{
+    // tile shapes whose rows share one block row: 128-row tiles, and 256-row ones where the blocks are that tall
+    unsigned allowed = (1u << 5) | (1u << 6);
+    if (bell.block % 256 == 0) allowed |= (1u << 0) | (1u << 13);
+    const TilePlan p = plan_tile(m, kell, n, allowed);
+    switch (p.variant) {
+    case 0: return launch_ptile_bell<TileP2, AF, BF>(m, kell, n, values, b, out, bell, p.nsplit, p.split_all, p.rotate, wsp, stream);
+    case 5: return launch_ptile_bell<TileH3, AF, BF>(m, kell, n, values, b, out, bell, p.nsplit, p.split_all, p.rotate, wsp, stream);
+    case 6: return launch_ptile_bell<TileQ2, AF, BF>(m, kell, n, values, b, out, bell, p.nsplit, p.split_all, p.rotate, wsp, stream);
+    case 13:
+        if (!p2h_ok(kell, p.nsplit)) return hipErrorInvalidValue;
+        return launch_ptile_bell<TileP2h, AF, BF>(m, kell, n, values, b, out, bell, p.nsplit, p.split_all, p.rotate, wsp, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
 // ------------------------------------------------------------------ skinny
 template <class S, int AF, int BF>
 hipError_t launch_skinny_shape(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,

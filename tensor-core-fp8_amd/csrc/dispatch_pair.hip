@@ -9,4 +9,6 @@
 namespace fp8gemm_detail {
 template hipError_t dispatch<FP8GEMM_PAIR_A, FP8GEMM_PAIR_B>(int, int, int, const uint8_t *, const uint8_t *, void *, int, int, int,
                                                              const OutSpec &, Workspace &, hipStream_t);
+template hipError_t dispatch_bell<FP8GEMM_PAIR_A, FP8GEMM_PAIR_B>(int, int, int, const uint8_t *, const uint8_t *, float *, const BellSpec &,
+                                                                  Workspace &, hipStream_t);
 }  // namespace fp8gemm_detail

@@ -29,8 +29,13 @@ extern template hipError_t dispatch<1, 0>(int, int, int, const uint8_t *, const 
 extern template hipError_t dispatch<1, 1>(int, int, int, const uint8_t *, const uint8_t *, void *, int, int, int,
                                           const OutSpec &, Workspace &, hipStream_t);
 
+extern template hipError_t dispatch_bell<0, 0>(int, int, int, const uint8_t *, const uint8_t *, float *, const BellSpec &, Workspace &, hipStream_t);
+extern template hipError_t dispatch_bell<0, 1>(int, int, int, const uint8_t *, const uint8_t *, float *, const BellSpec &, Workspace &, hipStream_t);
+extern template hipError_t dispatch_bell<1, 0>(int, int, int, const uint8_t *, const uint8_t *, float *, const BellSpec &, Workspace &, hipStream_t);
+extern template hipError_t dispatch_bell<1, 1>(int, int, int, const uint8_t *, const uint8_t *, float *, const BellSpec &, Workspace &, hipStream_t);
+
 namespace {
-constexpr int kVersion = 102;
+constexpr int kVersion = 103;
 // What the work lists and the planner's constants are laid out for: MI355X as one partition,
 // 256 CUs in 8 XCDs of 32, workgroups handed to the XCDs round robin (id mod 8).  On another
 // partition mode every result is still right (the work list only decides who computes what);
@@ -321,19 +326,20 @@ constexpr size_t kMaxSplitScratch = (size_t)1 << 30;
 // MFMA, whose one step takes 128 bytes of K, a 4-deep ring of 64-byte K tiles and a 2-deep ring of
 // 128-byte ones are the same pipeline; 4-deep rings of 64-byte K tiles under the 32x32x64 MFMA
 // measured 5 to 11 % slower than the 2- and 3-deep rings of 128-byte K tiles on every shape class.
-TilePlan plan_tile(int m, int k, int n)
+TilePlan plan_tile(int m, int k, int n, unsigned allowed)
 {
     TilePlan best = {0, 1, 2, false};
     const int kt = (k + 127) / 128;
     double best_cost = 1e30;
     for (const PtileCost &c : kPtileCosts) {
+        if (!((allowed >> c.variant) & 1u)) continue;
         // the 256 x 128 tile pays off where it holds all rows of A at once (no second
         // row of tiles re-reading the same B rows) and is at least half full
         if (c.variant == 8 && (m <= 128 || m > 256)) continue;
         // the weight-streaming tiles: one row of tiles, whole 128-byte K tiles
         if ((c.variant == 15 || c.variant == 16) && (m > c.bm || k % 128 != 0)) continue;
         // ... and up to 64 rows nothing else comes close to them
-        if (m <= 64 && k % 128 == 0 && c.variant != 15) continue;
+        if (m <= 64 && k % 128 == 0 && c.variant != 15 && ((allowed >> 15) & 1u)) continue;
         // overhanging K tile: only the shapes compiled for it
         if (k % 128 != 0 && !(c.variant == 0 || c.variant == 5 || c.variant == 6 || c.variant == 13 || c.variant == 14)) continue;
         for (int mode = 0; mode < 2; ++mode)          // 0: slices for the tail tiles only, 1: for all
@@ -453,15 +459,53 @@ hipError_t launch_spmm_bell(int m, int k, int n, int block, int ell_cols, const 
 }
 
 template <int SF, int XF>
-hipError_t launch_spmv_csr(int m, const uint8_t *values, const int *row_offsets, const int *col, const int *row_order,
+hipError_t launch_spmv_csr(int m, int k, const uint8_t *values, const int *row_offsets, const int *col, const int *row_order,
                            const uint8_t *x, float *y, hipStream_t stream)
 {
-    hipLaunchKernelGGL((spmv_csr_kernel<SF, XF>), dim3((unsigned)((m + 3) / 4)), dim3(256), 0, stream, m, values, row_offsets,
-                       col, row_order, x, y);
+    // 16-byte loads of the indices need the arrays aligned; up to 2048 waves walk the rows
+    const bool vec = reinterpret_cast<uintptr_t>(col) % 16 == 0 && reinterpret_cast<uintptr_t>(values) % 4 == 0;
+    if (!vec) {
+        hipLaunchKernelGGL((spmv_csr_kernel<SF, XF>), dim3((unsigned)((m + 3) / 4)), dim3(256), 0, stream, m, values, row_offsets,
+                           col, row_order, x, y);
+        return hipGetLastError();
+    }
+    // (workgroups of four waves; a wave walks a few rows, and some thirty waves per CU keep enough loads in flight)
+    const int groups = (m + 7) / 8 < 2048 ? (m + 7) / 8 : 2048;
+    if (k <= kSpmvLdsBytes) {
+        const int lds = (k + 15) / 16 * 16;
+        hipLaunchKernelGGL((spmv_csr_vec_kernel<SF, XF, true>), dim3((unsigned)groups), dim3(256), lds, stream, m, k, values,
+                           row_offsets, col, row_order, x, y);
+    } else {
+        hipLaunchKernelGGL((spmv_csr_vec_kernel<SF, XF, false>), dim3((unsigned)groups), dim3(256), 0, stream, m, k, values,
+                           row_offsets, col, row_order, x, y);
+    }
+    return hipGetLastError();
+}
+
+template <int SF, int XF>
+hipError_t launch_spmv_bell(int m, int k, int block, int ell_cols, const uint8_t *values, const int *block_cols,
+                            const uint8_t *x, float *y, hipStream_t stream)
+{
+    int shift = -1;
+    for (int b = 4; b < 31; ++b)
+        if (block == (1 << b)) shift = b;
+    // few 16-row groups: two or four waves share the K steps of a group, so that about 2048 waves run
+    const int groups16 = m / 16, steps = (ell_cols * block + 127) / 128;
+    int ksplit = groups16 >= 2048 ? 1 : (groups16 >= 1024 ? 2 : 4);
+    while (ksplit > 1 && steps < 4 * ksplit) ksplit /= 2;
+    const int per_wg = 4 / ksplit;
+    int grid = (groups16 + per_wg - 1) / per_wg;
+    if (ksplit == 1 && grid > 512) grid = 512;
+    hipLaunchKernelGGL((spmv_bell_kernel<SF, XF>), dim3((unsigned)grid), dim3(256), (k + 15) / 16 * 16 + 4096, stream, m, k, block,
+                       shift, ell_cols, ksplit, values, block_cols, x, y);
     return hipGetLastError();
 }
 
 bool fmt_ok(int f) { return f == FP8GEMM_E4M3 || f == FP8GEMM_E5M2; }
+
+// the tiled kernel's tiles are 128 rows or more and its K tiles 128 bytes; below 64 columns of
+// output a 128-column tile is mostly empty
+bool bell_tiled(int block, int n) { return block % 128 == 0 && n >= 64; }
 
 }  // namespace
 
@@ -492,6 +536,35 @@ int fp8gemm_spmm_bell(int m, int k, int n, int block, int ell_cols, const void *
     hipStream_t s = static_cast<hipStream_t>(stream);
     (void)hipGetLastError();
     hipError_t e;
+    // Blocks that hold whole 128-byte K tiles and whole 128-row tiles go through the LDS-tiled
+    // persistent kernel (the stored values are its A, the block list steers where the K tiles of
+    // B come from); other block sizes, and outputs of a few columns, through the direct kernel.
+    if (bell_tiled(block, n)) {
+        const BellSpec bell = {block_cols, ell_cols, block, k};
+        const int kell = ell_cols * block;
+        Workspace wsp = Workspace::pooled(s);
+        if (s_fmt == FP8GEMM_E4M3 && b_fmt == FP8GEMM_E4M3)
+            e = dispatch_bell<0, 0>(m, kell, n, pv, pb, out, bell, wsp, s);
+        else if (s_fmt == FP8GEMM_E5M2 && b_fmt == FP8GEMM_E5M2)
+            e = dispatch_bell<1, 1>(m, kell, n, pv, pb, out, bell, wsp, s);
+        else if (s_fmt == FP8GEMM_E4M3)
+            e = dispatch_bell<0, 1>(m, kell, n, pv, pb, out, bell, wsp, s);
+        else
+            e = dispatch_bell<1, 0>(m, kell, n, pv, pb, out, bell, wsp, s);
+        return (int)e;
+    }
+    if (n == 1 && k <= kSpmvLdsBytes) {
+        // matrix-vector: x fits LDS
+        if (s_fmt == FP8GEMM_E4M3 && b_fmt == FP8GEMM_E4M3)
+            e = launch_spmv_bell<0, 0>(m, k, block, ell_cols, pv, block_cols, pb, out, s);
+        else if (s_fmt == FP8GEMM_E5M2 && b_fmt == FP8GEMM_E5M2)
+            e = launch_spmv_bell<1, 1>(m, k, block, ell_cols, pv, block_cols, pb, out, s);
+        else if (s_fmt == FP8GEMM_E4M3)
+            e = launch_spmv_bell<0, 1>(m, k, block, ell_cols, pv, block_cols, pb, out, s);
+        else
+            e = launch_spmv_bell<1, 0>(m, k, block, ell_cols, pv, block_cols, pb, out, s);
+        return (int)e;
+    }
     if (s_fmt == FP8GEMM_E4M3 && b_fmt == FP8GEMM_E4M3)
         e = launch_spmm_bell<0, 0>(m, k, n, block, ell_cols, pv, block_cols, pb, out, s);
     else if (s_fmt == FP8GEMM_E5M2 && b_fmt == FP8GEMM_E5M2)
@@ -519,13 +592,13 @@ int fp8gemm_spmv_csr(int m, int k, const void *values, int s_fmt, const int *row
     (void)hipGetLastError();
     hipError_t e;
     if (s_fmt == FP8GEMM_E4M3 && x_fmt == FP8GEMM_E4M3)
-        e = launch_spmv_csr<0, 0>(m, pv, row_offsets, col_idx, row_order, px, y, s);
+        e = launch_spmv_csr<0, 0>(m, k, pv, row_offsets, col_idx, row_order, px, y, s);
     else if (s_fmt == FP8GEMM_E5M2 && x_fmt == FP8GEMM_E5M2)
-        e = launch_spmv_csr<1, 1>(m, pv, row_offsets, col_idx, row_order, px, y, s);
+        e = launch_spmv_csr<1, 1>(m, k, pv, row_offsets, col_idx, row_order, px, y, s);
     else if (s_fmt == FP8GEMM_E4M3)
-        e = launch_spmv_csr<0, 1>(m, pv, row_offsets, col_idx, row_order, px, y, s);
+        e = launch_spmv_csr<0, 1>(m, k, pv, row_offsets, col_idx, row_order, px, y, s);
     else
-        e = launch_spmv_csr<1, 0>(m, pv, row_offsets, col_idx, row_order, px, y, s);
+        e = launch_spmv_csr<1, 0>(m, k, pv, row_offsets, col_idx, row_order, px, y, s);
     return (int)e;
 }
 
@@ -552,11 +625,17 @@ int fp8gemm_spmm_csr(int m, int k, int n, const void *values, int s_fmt, const i
     if (e != hipSuccess) return (int)e;
     uint8_t *dense = static_cast<uint8_t *>(p) + kSliceCounterBytes;
     (void)hipGetLastError();
-    const size_t count16 = dense_bytes / 16;
-    hipLaunchKernelGGL(zero_bytes16_kernel, dim3((unsigned)((count16 + 255) / 256)), dim3(256), 0, s,
-                       reinterpret_cast<v4i *>(dense), count16);
-    hipLaunchKernelGGL(csr_densify_kernel, dim3((unsigned)((m + 3) / 4)), dim3(256), 0, s, m, (size_t)k,
-                       static_cast<const uint8_t *>(values), row_offsets, col_idx, dense);
+    if (k % 16 == 0 && k <= kSpmvLdsBytes) {
+        // a row at a time through LDS: one pass, whole 16-byte pieces out
+        hipLaunchKernelGGL(csr_densify_rows_kernel, dim3((unsigned)(m < 4096 ? m : 4096)), dim3(256), k, s, m, k,
+                           static_cast<const uint8_t *>(values), row_offsets, col_idx, dense);
+    } else {
+        const size_t count16 = dense_bytes / 16;
+        hipLaunchKernelGGL(zero_bytes16_kernel, dim3((unsigned)((count16 + 255) / 256)), dim3(256), 0, s,
+                           reinterpret_cast<v4i *>(dense), count16);
+        hipLaunchKernelGGL(csr_densify_kernel, dim3((unsigned)((m + 3) / 4)), dim3(256), 0, s, m, (size_t)k,
+                           static_cast<const uint8_t *>(values), row_offsets, col_idx, dense);
+    }
     e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
     Workspace gemm_ws = Workspace::fixed(gemm_bytes ? dense + dense_bytes : nullptr, gemm_bytes, false);

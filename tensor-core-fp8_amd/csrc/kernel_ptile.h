@@ -120,18 +120,20 @@ constexpr bool ptile_sums_slices_in_kernel = S::BM * S::BN <= 128 * 128;
 // common case carries no test for it.  EX: the output goes through `spec` (scale, fp32 /
 // bf16 / fp16); without it C receives the bare fp32 sums and `spec` is ignored.  BSTREAM: B is
 // loaded with the non-temporal hint (for a C with a single row of tiles, where every byte of B
-// is read by exactly one workgroup).
-template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM>
-__global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, int N,
-                                                                 const uint8_t *__restrict__ A,
-                                                                 const uint8_t *__restrict__ B,
-                                                                 void *__restrict__ C,
-                                                                 float *__restrict__ ws,
-                                                                 int *__restrict__ counters,
-                                                                 int tiles_m, int tiles_n, int GM, int CB,
-                                                                 int bulk, int tail, int nsplit,
-                                                                 int rounds, int rotate_and_skew, OutSpec spec)
+// is read by exactly one workgroup).  BELL: A is sparse in blocked-ELL form (`bell`).
+template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM, bool BELL>
+__device__ __forceinline__ void gemm_ptile_body(int M, int K, int N,
+                                                const uint8_t *__restrict__ A,
+                                                const uint8_t *__restrict__ B,
+                                                void *__restrict__ C,
+                                                float *__restrict__ ws,
+                                                int *__restrict__ counters,
+                                                int tiles_m, int tiles_n, int GM, int CB,
+                                                int bulk, int tail, int nsplit,
+                                                int rounds, int rotate_and_skew, OutSpec spec, BellSpec bell)
 {
+    static_assert(!BELL || (!KOVER && !BSTREAM), "the blocked-ELL form has whole K tiles and shares B between tile rows");
+    const int KB = BELL ? bell.kb : K;             // row stride of B
     const int rotate = rotate_and_skew & 0xFF;
     const int skew = rotate_and_skew >> 8;
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, CH = S::CH, RPI = S::RPI;
@@ -237,7 +239,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         const int jj = j < S::A_LOADS ? j : j - S::A_LOADS;
         const int per = j < S::A_LOADS ? S::A_LOADS : S::B_LOADS;
         const int row = (wave * per + jj) * RPI + lrow;
-        ld_off[j] = (uint32_t)row * (uint32_t)K + (uint32_t)((lslot ^ tile_swizzle<BK, S::SWZ>(row)) * 16);
+        ld_off[j] = (uint32_t)row * (uint32_t)(j < S::A_LOADS ? K : KB) + (uint32_t)((lslot ^ tile_swizzle<BK, S::SWZ>(row)) * 16);
     }
     const uint32_t ldsA = lds_base + (uint32_t)(wave * S::A_LOADS * RPI * BK);
     const uint32_t ldsB = lds_base + (uint32_t)(BM * BK + wave * S::B_LOADS * RPI * BK);
@@ -261,7 +263,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         if (q < nb) {
             int row = tile_n_ * BN + bpart * nb + q;
             row = row < N ? row : N - 1;
-            p = B + (size_t)row * K;
+            p = B + (size_t)row * KB;
         } else if (q - nb < na) {
             int row = tile_m_ * BM + apart * na + (q - nb);
             row = row < M ? row : M - 1;
@@ -278,18 +280,42 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
     // must then be small enough to stay in L2), rotate == 2 every XCD in every round (all
     // sharing inside an XCD is kept), 0 leaves the walk alone.
     int kt_base = 0, kt_rot = 0, kt_count = 1;
+    // Blocked-ELL A: where in B's rows each K tile of the planned item's walk lies.  Lane l of bell_at
+    // holds that byte offset for walk step 64 * bell_chunk + l (-1: a padding block), so the K loop
+    // gets it with v_readlane_b32 and no memory access; a fresh set of 64 is fetched when the walk
+    // crosses into the next chunk (a vector load whose wait drains the ring once per 64 K tiles).
+    const int *bell_row = nullptr;                 // block column list of the planned item's block row
+    int bell_at = -1, bell_chunk = -1;
+    uint32_t bell_koff = 0;                        // ... of the K tile being loaded
+    bool bell_pad = false;                         // ... or that it is a padding block
+    auto bell_fetch = [&](int chunk) __attribute__((always_inline)) {
+        const int tt = chunk * 64 + lane;
+        int v = -1;
+        if (tt < kt_count) {
+            int kk = tt + kt_rot;
+            kk = kk >= kt_count ? kk - kt_count : kk;
+            const int pos = (kt_base + kk) * BK;                    // byte position in the stored row
+            const int blk = pos / bell.block;
+            const int c = bell_row[blk];
+            v = c < 0 ? -1 : c * bell.block + (pos - blk * bell.block);
+        }
+        bell_at = v;
+        bell_chunk = chunk;
+    };
     auto plan_loads = [&](int tile_m, int tile_n, int kt0, int count, int item) __attribute__((always_inline)) {
         const int m0 = tile_m * BM, n0 = tile_n * BN;
         const int rows_a = M - m0 < BM ? M - m0 : BM;
         const int rows_b = N - n0 < BN ? N - n0 : BN;
         rsA = make_buffer_resource(A + (size_t)m0 * K, (unsigned long long)rows_a * (unsigned long long)K);
-        rsB = make_buffer_resource(B + (size_t)n0 * K, (unsigned long long)rows_b * (unsigned long long)K);
+        rsB = make_buffer_resource(B + (size_t)n0 * KB, (unsigned long long)rows_b * (unsigned long long)KB);
+        if constexpr (BELL) bell_row = bell.cols + (size_t)(m0 / bell.block) * bell.ell_cols;
         kt_base = kt0;
         kt_count = count;
         const unsigned key = rotate == 1 ? (unsigned)tile_n : (unsigned)item;   // item: (round, XCD)
         // (the division runs on the vector unit; the result is the same in every lane)
         kt_rot = rotate == 0 ? 0 : __builtin_amdgcn_readfirstlane((int)(((key * 2654435761u) >> 8) % (unsigned)count));
         plan_prefetch(tile_m, tile_n, items_in_xcd);
+        if constexpr (BELL) bell_fetch(0);
     };
     // load number j (0 .. LOADS-1) of step `ktile` of the planned item's K walk into ring slot `stage`
     // (the lambdas around the loads are forced inline: a closure left in memory would turn the
@@ -309,6 +335,20 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
             const uint32_t kpos = koff + (uint32_t)((lslot ^ tile_swizzle<BK, S::SWZ>(row)) * 16);
             voff = kpos >= (uint32_t)K ? 0xFFFFFFF0u : voff;
         }
+        if constexpr (BELL) {
+            if (j == S::A_LOADS) {                 // first load of B of this K tile: where its block lies
+                if ((ktile >> 6) != bell_chunk) bell_fetch(ktile >> 6);               // (uniform, once per 64 K tiles)
+                const int at = __builtin_amdgcn_readlane(bell_at, ktile & 63);
+                bell_pad = at < 0;
+                bell_koff = (uint32_t)at;
+            }
+            if (j >= S::A_LOADS) {
+                // a padding block: every lane's address goes outside the extent and reads zeros
+                buffer_load_lds_b128(rsB, ldsB + sbase + (uint32_t)((j - S::A_LOADS) * RPI * BK), bell_pad ? 0xFFFFFFF0u : voff,
+                                     bell_pad ? 0u : bell_koff);
+                return;
+            }
+        }
         if (j < S::A_LOADS)
             buffer_load_lds_b128(rsA, ldsA + sbase + (uint32_t)(j * RPI * BK), voff, koff);
         else if (BSTREAM)
@@ -324,7 +364,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
     // (a load that writes LDS, into 256 bytes past everything else that nobody reads: a load
     // into a register would write that register whenever it returns, behind the compiler's back)
     auto issue_prefetch = [&](int ktile) __attribute__((always_inline)) {
-        if constexpr (BSTREAM) return;
+        if constexpr (BSTREAM || BELL) return;
         int kk = ktile < kt_count ? ktile : kt_count - 1;
         kk += kt_rot;
         kk = kk >= kt_count ? kk - kt_count : kk;
@@ -338,7 +378,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
     // shapes whose operands stay in the caches are unchanged).  Not where B streams past with the
     // non-temporal hint (one row of tiles: M=256 N=28672 K=8192 76 -> 84 us with the prefetch):
     // there every line is used once, by one workgroup, and asking for it twice only adds requests.
-    constexpr int NPF = BSTREAM ? 0 : 1;
+    constexpr int NPF = (BSTREAM || BELL) ? 0 : 1;
     constexpr int pf_dist = 1;
 
     // Start skew: the workgroups of an XCD that work on tile row i of its window start i * skew
@@ -811,6 +851,38 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
         T = next_T;
         ws_slot = next_ws_slot;
     }
+}
+
+template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM>
+__global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, int N,
+                                                                 const uint8_t *__restrict__ A,
+                                                                 const uint8_t *__restrict__ B,
+                                                                 void *__restrict__ C,
+                                                                 float *__restrict__ ws,
+                                                                 int *__restrict__ counters,
+                                                                 int tiles_m, int tiles_n, int GM, int CB,
+                                                                 int bulk, int tail, int nsplit,
+                                                                 int rounds, int rotate_and_skew, OutSpec spec)
+{
+    gemm_ptile_body<S, AF, BF, KOVER, EX, BSTREAM, false>(M, K, N, A, B, C, ws, counters, tiles_m, tiles_n, GM, CB, bulk, tail,
+                                                          nsplit, rounds, rotate_and_skew, spec, BellSpec{nullptr, 0, 0, 0});
+}
+
+// The same kernel with A in blocked-ELL form: out = S * B^T, S stored as `A` (M x K values) and `bell`.
+template <class S, int AF, int BF>
+__global__ __launch_bounds__(S::THREADS) void gemm_ptile_bell_kernel(int M, int K, int N,
+                                                                      const uint8_t *__restrict__ A,
+                                                                      const uint8_t *__restrict__ B,
+                                                                      void *__restrict__ C,
+                                                                      float *__restrict__ ws,
+                                                                      int *__restrict__ counters,
+                                                                      int tiles_m, int tiles_n, int GM, int CB,
+                                                                      int bulk, int tail, int nsplit,
+                                                                      int rounds, int rotate_and_skew, BellSpec bell)
+{
+    const OutSpec plain = {1.0f, nullptr, nullptr, FP8GEMM_DEV_OUT_F32, 0.0f, nullptr, FP8GEMM_DEV_OUT_F32, nullptr, nullptr, nullptr};
+    gemm_ptile_body<S, AF, BF, false, false, false, true>(M, K, N, A, B, C, ws, counters, tiles_m, tiles_n, GM, CB, bulk, tail,
+                                                          nsplit, rounds, rotate_and_skew, plain, bell);
 }
 
 #endif  // FP8GEMM_KERNEL_PTILE_H

@@ -114,6 +114,92 @@ __global__ __launch_bounds__(64) void spmm_bell_kernel(int m, int k, int n, int 
     }
 }
 
+// Matrix-vector product with S in blocked-ELL form, x (k codes, k <= kSpmvLdsBytes) held in LDS.
+// Bound by reading the stored values once: every wave keeps the loads of DEPTH K steps in flight
+// (the values of a step and the block columns its pieces need) and takes the pieces of x from
+// LDS.  The MFMA multiplies 16 rows of S by 16 copies of x; column 0 is stored.  Lane roles as in
+// spmm_bell_kernel.  Two ways of handing out the work, chosen by the host through `ksplit`:
+//   1: many rows -- the four waves of a workgroup each walk 16-row groups (g, g + waves, ..);
+//   2 or 4: few rows -- that many waves share a group, wave u of them taking K steps u,
+//      u + ksplit, ..; their sums meet in LDS and are added in the order of u.  One pass, the
+//      grid covers every group.
+constexpr int kSpmvLdsBytes = 60 * 1024;       // with the 4 KiB for the sums: the 64 KiB of LDS a kernel gets without asking
+
+template <int SF, int XF>
+__global__ __launch_bounds__(256) void spmv_bell_kernel(int m, int k, int block, int block_shift, int ell_cols, int ksplit,
+                                                         const uint8_t *__restrict__ values,
+                                                         const int *__restrict__ block_cols,
+                                                         const uint8_t *__restrict__ x, float *__restrict__ y)
+{
+    constexpr int DEPTH = 4;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_x[];      // x, then 4 KiB for the waves' sums
+    const int xbytes = (k + 15) & ~15;
+    for (int t = threadIdx.x * 16; t < k; t += 256 * 16) *reinterpret_cast<v4i *>(lds_x + t) = load_piece(x + t);
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = lane & 15, q = lane >> 4;
+    const int kell = ell_cols * block;
+    const int steps = (kell + 127) / 128;
+    const int groups = m / 16;
+    const v4i zero = {0, 0, 0, 0};
+    const int sub = wave % ksplit;                                      // which share of the K steps
+    const int per_wg = 4 / ksplit;                                      // groups a workgroup has at a time
+    const int stride = ksplit == 1 ? gridDim.x * 4 : groups;            // (ksplit > 1: a single pass)
+    for (int g = blockIdx.x * per_wg + wave / ksplit; g < groups || ksplit > 1; g += stride) {
+        const bool have = g < groups;
+        v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        const int row0 = have ? g * 16 : 0;
+        if (have) {
+            const int *cols = block_cols + (size_t)(row0 / block) * ell_cols;
+            const uint8_t *srow = values + (size_t)(row0 + i) * kell;
+            const int mine = (steps - sub + ksplit - 1) / ksplit;       // K steps sub, sub + ksplit, ..
+            v4i a[DEPTH][2];
+            int at[DEPTH][2];      // where in x the piece lies; -1: nowhere (padding block, or past the stored row)
+            auto fetch = [&](int u, int d) __attribute__((always_inline)) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int p = (sub + u * ksplit) * 128 + (2 * q + h) * 16;
+                    a[d][h] = zero;
+                    at[d][h] = -1;
+                    if (p < kell) {
+                        const int blk = block_shift >= 0 ? p >> block_shift : p / block;
+                        const int c = cols[blk];
+                        a[d][h] = load_piece(srow + p);
+                        at[d][h] = c < 0 ? -1 : c * block + (p - blk * block);
+                    }
+                }
+            };
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d)
+                if (d < mine) fetch(d, d);
+            for (int u0 = 0; u0 < mine; u0 += DEPTH) {
+#pragma unroll
+                for (int d = 0; d < DEPTH; ++d) {
+                    if (u0 + d < mine) {                               // (uniform)
+                        v4i xp[2];
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) xp[h] = at[d][h] >= 0 ? *reinterpret_cast<const v4i *>(lds_x + at[d][h]) : zero;
+                        acc = mfma_16x16x128<SF, XF>(pack8(a[d][0], a[d][1]), pack8(xp[0], xp[1]), acc);
+                        if (u0 + d + DEPTH < mine) fetch(u0 + d + DEPTH, d);
+                    }
+                }
+            }
+        }
+        if (ksplit > 1) {
+            v4f *sums = reinterpret_cast<v4f *>(lds_x + xbytes);
+            sums[wave * 64 + lane] = acc;
+            __syncthreads();
+            if (sub == 0)
+                for (int u = 1; u < ksplit; ++u) acc += sums[(wave + u) * 64 + lane];
+        }
+        if (have && sub == 0 && i == 0) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) y[row0 + 4 * q + r] = acc[r];
+        }
+        if (ksplit > 1) break;
+    }
+}
+
 // y[row] = sum over the stored entries of the row of float(values[e]) * float(x[col[e]]):
 // one wave per row, in the order row_order gives (null: 0, 1, 2, ..; the reference's
 // SortedRowSwizzle, bm_test_utils.h:202-216, puts the longest rows first so that they start
@@ -138,6 +224,82 @@ __global__ __launch_bounds__(256) void spmv_csr_kernel(int m, const uint8_t *__r
     if (lane == 0) y[row] = acc;
 }
 
+// The same with 16-byte loads of the indices and 4-byte loads of the values (four entries per lane
+// and pass, two passes in flight), waves that walk a few rows each (row w, w + waves, ..), and x in LDS
+// (XLDS: k <= kSpmvLdsBytes; otherwise x is gathered through the caches).  A row's entries are taken in
+// aligned groups of four starting at the group that holds its first entry; entries of the neighbouring
+// rows in the first and last group are masked out, and the last groups of the arrays are read
+// element by element, so nothing past the arrays' ends is touched.
+// Requirements checked by the host: col 16-byte aligned, values 4-byte aligned.
+template <int SF, int XF, bool XLDS>
+__global__ __launch_bounds__(256) void spmv_csr_vec_kernel(int m, int k, const uint8_t *__restrict__ values,
+                                                            const int *__restrict__ row_offsets,
+                                                            const int *__restrict__ col,
+                                                            const int *__restrict__ row_order,
+                                                            const uint8_t *__restrict__ x, float *__restrict__ y)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_x[];
+    if (XLDS) {
+        // (k need not be a multiple of 16: the tail goes byte by byte)
+        const int k16 = k & ~15;
+        const bool aligned = reinterpret_cast<uintptr_t>(x) % 16 == 0;
+        if (aligned)
+            for (int t = threadIdx.x * 16; t < k16; t += 256 * 16) *reinterpret_cast<v4i *>(lds_x + t) = load_piece(x + t);
+        for (int t = (aligned ? k16 : 0) + threadIdx.x; t < k; t += 256) lds_x[t] = x[t];
+        __syncthreads();
+    }
+    const uint8_t *xs = XLDS ? lds_x : x;
+    const int lane = threadIdx.x & 63;
+    const int waves = gridDim.x * 4;
+    const int nnz = row_offsets[m];
+    const int vec_end = nnz & ~3;                 // groups of four that lie wholly inside the arrays
+    int w = blockIdx.x * 4 + (threadIdx.x >> 6);
+    int row = 0, e0 = 0, e1 = 0;
+    if (w < m) {
+        row = row_order ? row_order[w] : w;
+        e0 = row_offsets[row];
+        e1 = row_offsets[row + 1];
+    }
+    while (w < m) {
+        // the next row's bounds are on their way while this row is added up
+        const int wn = w + waves;
+        int rown = 0, e0n = 0, e1n = 0;
+        if (wn < m) {
+            rown = row_order ? row_order[wn] : wn;
+            e0n = row_offsets[rown];
+            e1n = row_offsets[rown + 1];
+        }
+        float acc = 0.0f;
+        auto one = [&](int e) __attribute__((always_inline)) {
+            if (e >= e0 && e < e1) acc += fp8_to_float<SF>(values[e]) * fp8_to_float<XF>(xs[col[e]]);
+        };
+        auto four = [&](int e) __attribute__((always_inline)) {
+            if (e + 4 <= vec_end) {
+                const v4i c4 = *reinterpret_cast<const v4i *>(col + e);
+                const uint32_t v4 = *reinterpret_cast<const uint32_t *>(values + e);
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    if (e + t >= e0 && e + t < e1) acc += fp8_to_float<SF>((v4 >> (8 * t)) & 0xFFu) * fp8_to_float<XF>(xs[c4[t]]);
+            } else {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    if (e + t < nnz) one(e + t);
+            }
+        };
+        for (int e = (e0 & ~3) + lane * 4; e < e1; e += 512) {
+            four(e);
+            if (e + 256 < e1) four(e + 256);
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+        if (lane == 0) y[row] = acc;
+        w = wn;
+        row = rown;
+        e0 = e0n;
+        e1 = e1n;
+    }
+}
+
 // dense[0 .. count16) = 0, 16 bytes per thread
 __global__ __launch_bounds__(256) void zero_bytes16_kernel(v4i *__restrict__ dense, size_t count16)
 {
@@ -160,6 +322,30 @@ __global__ __launch_bounds__(256) void csr_densify_kernel(int m, size_t ld, cons
     for (int e = row_offsets[row] + lane; e < e1; e += 64) {
         const uint8_t v = values[e];
         if ((v & 0x7F) != 0) dense[(size_t)row * ld + col[e]] = v;
+    }
+}
+
+// The same in one pass for rows of up to kSpmvLdsBytes bytes (k % 16 == 0): a workgroup builds a
+// row of the dense matrix in LDS -- zeros, then the row's stored entries -- and writes it out in
+// whole 16-byte pieces; `dense` need not hold zeros.
+__global__ __launch_bounds__(256) void csr_densify_rows_kernel(int m, int k, const uint8_t *__restrict__ values,
+                                                                const int *__restrict__ row_offsets,
+                                                                const int *__restrict__ col, uint8_t *__restrict__ dense)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_row[];
+    const v4i zero = {0, 0, 0, 0};
+    for (int row = blockIdx.x; row < m; row += gridDim.x) {
+        for (int t = threadIdx.x * 16; t < k; t += 256 * 16) *reinterpret_cast<v4i *>(lds_row + t) = zero;
+        __syncthreads();
+        const int e1 = row_offsets[row + 1];
+        for (int e = row_offsets[row] + threadIdx.x; e < e1; e += 256) {
+            const uint8_t v = values[e];
+            if ((v & 0x7F) != 0) lds_row[col[e]] = v;
+        }
+        __syncthreads();
+        for (int t = threadIdx.x * 16; t < k; t += 256 * 16)
+            *reinterpret_cast<v4i *>(dense + (size_t)row * k + t) = *reinterpret_cast<const v4i *>(lds_row + t);
+        __syncthreads();
     }
 }
 

@@ -55,7 +55,8 @@ struct TilePlan {
     int variant, nsplit, rotate;
     bool split_all;      // K slices for every tile (else only for the tiles that do not fill a round)
 };
-TilePlan plan_tile(int m, int k, int n);
+// allowed: bit v set = tile shape number v may be picked
+TilePlan plan_tile(int m, int k, int n, unsigned allowed = ~0u);
 size_t tile_plan_scratch_bytes(int m, int n, const TilePlan &p);
 
 // Where the partial sums of one call's K slices go: a buffer of the per-(device, stream)
@@ -95,6 +96,12 @@ hipError_t launch_tile_slices_reduce(const float *ws, void *out, int m, int n, i
 template <int AF, int BF>
 hipError_t dispatch(int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
                     int algo, int variant, int nsplit, const OutSpec &spec, Workspace &wsp, hipStream_t stream);
+
+// The same for a sparse A in blocked-ELL form whose blocks hold whole tiles (block % 128 == 0):
+// `values` is the m x kell matrix of stored values, `bell` the block list and B's row stride.
+template <int AF, int BF>
+hipError_t dispatch_bell(int m, int kell, int n, const uint8_t *values, const uint8_t *b, float *out, const BellSpec &bell,
+                         Workspace &wsp, hipStream_t stream);
 
 }  // namespace fp8gemm_detail
 

@@ -66,6 +66,44 @@ def test_spmm_bell_all_finite_codes(pkg, oracle, fs, fb, block, ell, m, k, n):
 
 
 @pytest.mark.parametrize("fs,fb", PAIRS)
+@pytest.mark.parametrize("block,ell,m,k,n", [(128, 4, 512, 4096, 300), (256, 2, 512, 2048, 256), (128, 40, 256, 8192, 512),
+                                              (256, 16, 1024, 8192, 1024), (128, 1, 128, 128, 64), (384, 2, 768, 1536, 200),
+                                              (128, 3, 2304, 2048, 2200)])
+def test_spmm_bell_through_the_tiled_kernel(pkg, oracle, fs, fb, block, ell, m, k, n):
+    """Blocks of whole 128-byte K tiles and whole tile rows run on the LDS-tiled persistent kernel:
+    128- and 256-row tiles, both MFMA shapes, K slices (few tiles, long stored rows), more tiles
+    than CUs with leftover tiles, a single K tile, padding blocks, n that overhangs the tile."""
+    rng = np.random.default_rng(zlib.crc32(repr(("tiled", fs, fb, block, ell, m, k, n)).encode()))
+    vals, bcols = random_bell(rng, m, k, block, ell, fs, pad_some=ell > 1)
+    B = random_codes(rng, (n, k), fb)
+    if fb == 1:
+        B = np.where(((B >> 2) & 0x1F) > 24, B & 0x83 | 0x3C, B).astype(np.uint8)
+    out = pkg.spmm_bell(dev(vals), dev(bcols), block, dev(B), k, s_fmt=fs, b_fmt=fb).cpu().numpy()
+    v, offs, col = oracle.bell_to_csr(vals, bcols, block)
+    ref, tol = bound(oracle, v, fs, offs, col, k, B, fb, mfma=True)
+    check(out, ref, tol)
+
+
+@pytest.mark.parametrize("fs,fb", PAIRS)
+@pytest.mark.parametrize("block", [128, 256])
+def test_spmm_bell_tiled_one_hot_is_bit_exact(pkg, oracle, fs, fb, block):
+    """The tiled kernel's gather through the block list, bit for bit: one value of 1.0 per row of S."""
+    one = {0: 0x38, 1: 0x3C}
+    ell, m, k, n = 3, 2 * block, 8 * block, 256
+    rng = np.random.default_rng(177 + fs + block)
+    _, bcols = random_bell(rng, m, k, block, ell, fs)
+    vals = np.zeros((m, ell * block), dtype=np.uint8)
+    pos = rng.integers(0, ell * block, m)
+    vals[np.arange(m), pos] = one[fs]
+    col = bcols[np.arange(m) // block, pos // block] * block + pos % block
+    codes = finite_codes(fb)
+    B = codes[rng.integers(0, codes.size, (n, k))]
+    B[:, col[0]] = np.resize(codes, n)
+    out = pkg.spmm_bell(dev(vals), dev(bcols), block, dev(B), k, s_fmt=fs, b_fmt=fb).cpu().numpy()
+    assert np.array_equal(out, oracle.decode(B, fb)[:, col].T)
+
+
+@pytest.mark.parametrize("fs,fb", PAIRS)
 def test_spmm_bell_normal_values_plain_bound(pkg, oracle, fs, fb):
     """N(0,1)-like values, long stored rows: the plain reordering bound, no hardware term."""
     rng = np.random.default_rng(31 + fs * 2 + fb)
