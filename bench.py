@@ -169,6 +169,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host CPU leg")
     ap.add_argument("--no-vendor", action="store_true", help="skip the hipBLASLt comparison (a child process)")
     ap.add_argument("--no-llm-shapes", action="store_true", help="time only M=16 N=28672 K=8192 of the skinny shapes")
+    ap.add_argument("--no-sparse", action="store_true", help="skip the SpMV / SpMM shapes")
     ap.add_argument("--no-more-shapes", action="store_true",
                     help="skip 16384^3, the four pairings at 4096^3 and the K=32768 stress shapes")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -405,6 +406,97 @@ def main():
               "note": "cold = rotating over %d weight buffers (nothing of the next one left in the 256 MB Infinity "
                       "Cache), warm = same buffer every launch" % head["weight_buffers"]}
 
+    # ---------------------------------------------------------------- sparse operands (SpMV: HBM-bound, SpMM: MFMA on stored blocks)
+    sparse = []
+    if not args.no_sparse:
+        rng = np.random.default_rng(0x5BA)
+
+        def raw_time(fn_of_i, steps2):
+            settle(torch, fn_of_i, block=50, cap_s=0.3)
+            return time_launches(torch, fn_of_i, steps2, 20)[0]
+
+        def ck(code):
+            if code != 0:
+                pkg.check(code)
+
+        # blocked-ELL: block columns as the reference's generator draws them (distinct, rising, uniform)
+        def bell_operand(m2, k2, block, ell):
+            cols = np.stack([np.sort(rng.permutation(k2 // block)[:ell]) for _ in range(m2 // block)]).astype(np.int32)
+            vals = pkg.fill((m2, ell * block), pkg.E4M3, seed=0x5BA + m2 + block, dist="normal")
+            return torch.from_numpy(vals).to(dev), torch.from_numpy(cols).to(dev)
+
+        # matrix-vector, blocked-ELL: pruned weight matrix 28672 x 8192, a quarter of the 64 x 64 blocks kept
+        m2, k2, block, ell = 28672, 8192, 64, 32
+        ncopy = 6
+        ops = [bell_operand(m2, k2, block, ell) for _ in range(ncopy)]
+        xv = torch.from_numpy(pkg.fill((k2,), pkg.E4M3, seed=0x5BA + 1, dist="normal")).to(dev)
+        yv = torch.empty(m2, dtype=torch.float32, device=dev)
+
+        def go_bell_mv(i):
+            v, c = ops[i % ncopy]
+            ck(L.fp8gemm_spmv_bell(m2, k2, block, ell, v.data_ptr(), 0, c.data_ptr(), xv.data_ptr(), 0, yv.data_ptr(), stream))
+        ms_c = raw_time(go_bell_mv, 120)
+        ms_w = raw_time(lambda i: go_bell_mv(0), 120)
+        by = m2 * ell * block + (m2 // block) * ell * 4 + k2 + 4 * m2
+        sparse.append({"kernel": "fp8gemm_spmv_bell", "M": m2, "K": k2, "block": block, "stored_blocks_per_row": ell,
+                       "density": ell * block / k2, "algorithmic_bytes": by, "us_cold": ms_c * 1e3, "us_warm": ms_w * 1e3,
+                       "gbs_cold": by / ms_c / 1e6, "frac_hbm_peak_cold": by / ms_c / 1e6 / PEAK_HBM_GBS, "copies_rotated": ncopy})
+        del ops
+
+        # matrix-vector, CSR: the same matrix shape, one element in ten kept at uniformly drawn places
+        mask = rng.random((m2, k2)) < 0.10
+        offs = np.concatenate([[0], np.cumsum(mask.sum(axis=1))]).astype(np.int32)
+        colh = np.nonzero(mask)[1].astype(np.int32)
+        del mask
+        nnz = int(offs[-1])
+        ncopy = 4
+        csr_ops = []
+        for c in range(ncopy):
+            csr_ops.append((torch.from_numpy(pkg.fill((nnz,), pkg.E4M3, seed=0x5BA + 7 + c, dist="normal")).to(dev),
+                            torch.from_numpy(offs).to(dev), torch.from_numpy(colh).to(dev)))
+
+        def go_csr_mv(i):
+            v, o, c = csr_ops[i % ncopy]
+            ck(L.fp8gemm_spmv_csr(m2, k2, v.data_ptr(), 0, o.data_ptr(), c.data_ptr(), None, xv.data_ptr(), 0, yv.data_ptr(), stream))
+        ms_c = raw_time(go_csr_mv, 120)
+        ms_w = raw_time(lambda i: go_csr_mv(0), 120)
+        by = 5 * nnz + 4 * (m2 + 1) + k2 + 4 * m2
+        sparse.append({"kernel": "fp8gemm_spmv_csr", "M": m2, "K": k2, "stored_entries": nnz, "density": nnz / (m2 * k2),
+                       "algorithmic_bytes": by, "us_cold": ms_c * 1e3, "us_warm": ms_w * 1e3, "gbs_cold": by / ms_c / 1e6,
+                       "frac_hbm_peak_cold": by / ms_c / 1e6 / PEAK_HBM_GBS, "copies_rotated": ncopy})
+        del csr_ops
+
+        # matrix-matrix, blocked-ELL, blocks of whole tiles (the LDS-tiled kernel) and small blocks (the direct kernel)
+        for (m3, k3, n3, block, ell) in [(8192, 8192, 8192, 256, 8), (8192, 8192, 8192, 128, 16), (4096, 4096, 4096, 32, 32)]:
+            v, c = bell_operand(m3, k3, block, ell)
+            Bd = torch.from_numpy(pkg.fill((n3, k3), pkg.E4M3, seed=0x5BA + 3, dist="normal")).to(dev)
+            Cd = torch.empty((m3, n3), dtype=torch.float32, device=dev)
+            ms3 = raw_time(lambda i: ck(L.fp8gemm_spmm_bell(m3, k3, n3, block, ell, v.data_ptr(), 0, c.data_ptr(), Bd.data_ptr(), 0,
+                                                            Cd.data_ptr(), stream)), 30)
+            fl = 2.0 * m3 * ell * block * n3
+            sparse.append({"kernel": "fp8gemm_spmm_bell", "M": m3, "K": k3, "N": n3, "block": block, "stored_blocks_per_row": ell,
+                           "density": ell * block / k3, "us": ms3 * 1e3, "tflops_on_stored_blocks": fl / ms3 / 1e9,
+                           "frac_of_fp8_peak_on_stored_blocks": fl / ms3 / 1e9 / PEAK_FP8_TFLOPS,
+                           "dense_equivalent_tflops": 2.0 * m3 * k3 * n3 / ms3 / 1e9})
+            del v, c, Bd, Cd
+        # matrix-matrix, CSR: through the dense scratch and the dense GEMM
+        m3 = k3 = n3 = 4096
+        mask = rng.random((m3, k3)) < 0.10
+        offs = np.concatenate([[0], np.cumsum(mask.sum(axis=1))]).astype(np.int32)
+        colh = np.nonzero(mask)[1].astype(np.int32)
+        nnz = int(offs[-1])
+        v = torch.from_numpy(pkg.fill((nnz,), pkg.E4M3, seed=0x5BA + 9, dist="normal")).to(dev)
+        o, c = torch.from_numpy(offs).to(dev), torch.from_numpy(colh).to(dev)
+        Bd = torch.from_numpy(pkg.fill((n3, k3), pkg.E4M3, seed=0x5BA + 3, dist="normal")).to(dev)
+        Cd = torch.empty((m3, n3), dtype=torch.float32, device=dev)
+        ms3 = raw_time(lambda i: ck(L.fp8gemm_spmm_csr(m3, k3, n3, v.data_ptr(), 0, o.data_ptr(), c.data_ptr(), Bd.data_ptr(), 0,
+                                                       Cd.data_ptr(), stream)), 30)
+        sparse.append({"kernel": "fp8gemm_spmm_csr", "M": m3, "K": k3, "N": n3, "stored_entries": nnz, "density": nnz / (m3 * k3),
+                       "us": ms3 * 1e3, "dense_equivalent_tflops": 2.0 * m3 * k3 * n3 / ms3 / 1e9,
+                       "note": "S is written out as a dense fp8 matrix in scratch, then the dense GEMM runs"})
+        del v, o, c, Bd, Cd, xv, yv
+        torch.cuda.empty_cache()
+
     # ---------------------------------------------------------------- CPU baseline (host cores)
     cpu = None
     if not args.no_cpu_baseline:
@@ -503,6 +595,7 @@ def main():
         "stress_k32768": stress_k32768,
         "skinny": skinny,
         "llm_shapes": llm,
+        "sparse": sparse,
         "parity": parity,
         "cpu_baseline": cpu,
         "vendor": vendor,

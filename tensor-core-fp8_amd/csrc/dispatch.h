@@ -59,7 +59,7 @@ hipError_t allow_lds(Kernel kernel, int bytes)
     return e;
 }
 
-template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM>
+template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM, bool NOPF = false>
 struct PtileKernelTag {};
 template <class S, int AF, int BF>
 struct SkinnyKernelTag {};
@@ -87,13 +87,13 @@ inline int start_skew(const PtileWork &w)
 
 // persistent form: one workgroup per CU walks its share of the work list; the K slices'
 // partial sums go through the scratch buffer and a reduction pass
-template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM>
+template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM, bool NOPF = false>
 hipError_t launch_ptile_work(const PtileWork &w, int m, int k, int n, const uint8_t *a, const uint8_t *b, void *out,
                              float *ws, int *counters, int rotate, const OutSpec &spec, hipStream_t stream)
 {
-    auto kernel = gemm_ptile_kernel<S, AF, BF, KOVER, EX, BSTREAM>;
+    auto kernel = gemm_ptile_kernel<S, AF, BF, KOVER, EX, BSTREAM, NOPF>;
     constexpr int kLdsBytes = S::PTILE_LDS_BYTES + 256 + 16;      // + the landing place of the L2 prefetches + a flag
-    hipError_t e = allow_lds<PtileKernelTag<S, AF, BF, KOVER, EX, BSTREAM>>(kernel, kLdsBytes);
+    hipError_t e = allow_lds<PtileKernelTag<S, AF, BF, KOVER, EX, BSTREAM, NOPF>>(kernel, kLdsBytes);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * w.slots)), dim3(S::THREADS), kLdsBytes, stream,
                        m, k, n, a, b, out, ws, counters, w.tiles_m, w.tiles_n, w.GM, tile_column_block(w.tiles_n, m, n, k), w.bulk, w.tail,
@@ -132,6 +132,15 @@ hipError_t launch_ptile_shape_k(int m, int k, int n, const uint8_t *a, const uin
         if (kSumInKernel && wsp.counters_zero() && w.tail <= kMaxSliceCounters && window_fits) counters = static_cast<int *>(p);
     }
     hipError_t e;
+    // the compute-bound tiles on operands that both stay in the last-level cache: no L2 prefetch (see the kernel)
+    const bool cached = (size_t)m * k + (size_t)n * k <= ((size_t)192 << 20);
+    if constexpr (S::MF16 && !KOVER && !EX) {
+        if (cached) {
+            e = launch_ptile_work<S, AF, BF, false, false, false, true>(w, m, k, n, a, b, out, ws, counters, rotate, spec, stream);
+            if (e != hipSuccess || w.nsplit == 1 || counters) return e;
+            return launch_tile_slices_reduce(base, out, m, n, k, S::BM, S::BN, w, spec, stream);
+        }
+    }
     if constexpr (STREAM_TOO && !KOVER) {
         e = w.tiles_m == 1 ? launch_ptile_work<S, AF, BF, KOVER, EX, true>(w, m, k, n, a, b, out, ws, counters, rotate, spec, stream)
                            : launch_ptile_work<S, AF, BF, KOVER, EX, false>(w, m, k, n, a, b, out, ws, counters, rotate, spec, stream);

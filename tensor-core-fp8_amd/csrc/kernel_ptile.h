@@ -120,8 +120,9 @@ constexpr bool ptile_sums_slices_in_kernel = S::BM * S::BN <= 128 * 128;
 // common case carries no test for it.  EX: the output goes through `spec` (scale, fp32 /
 // bf16 / fp16); without it C receives the bare fp32 sums and `spec` is ignored.  BSTREAM: B is
 // loaded with the non-temporal hint (for a C with a single row of tiles, where every byte of B
-// is read by exactly one workgroup).  BELL: A is sparse in blocked-ELL form (`bell`).
-template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM, bool BELL>
+// is read by exactly one workgroup).  BELL: A is sparse in blocked-ELL form (`bell`).  NOPF: without
+// the L2 prefetch (see NPF below).
+template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM, bool BELL, bool NOPF>
 __device__ __forceinline__ void gemm_ptile_body(int M, int K, int N,
                                                 const uint8_t *__restrict__ A,
                                                 const uint8_t *__restrict__ B,
@@ -364,7 +365,7 @@ __device__ __forceinline__ void gemm_ptile_body(int M, int K, int N,
     // (a load that writes LDS, into 256 bytes past everything else that nobody reads: a load
     // into a register would write that register whenever it returns, behind the compiler's back)
     auto issue_prefetch = [&](int ktile) __attribute__((always_inline)) {
-        if constexpr (BSTREAM || BELL) return;
+        if constexpr (BSTREAM || BELL || NOPF) return;
         int kk = ktile < kt_count ? ktile : kt_count - 1;
         kk += kt_rot;
         kk = kk >= kt_count ? kk - kt_count : kk;
@@ -378,7 +379,10 @@ __device__ __forceinline__ void gemm_ptile_body(int M, int K, int N,
     // shapes whose operands stay in the caches are unchanged).  Not where B streams past with the
     // non-temporal hint (one row of tiles: M=256 N=28672 K=8192 76 -> 84 us with the prefetch):
     // there every line is used once, by one workgroup, and asking for it twice only adds requests.
-    constexpr int NPF = (BSTREAM || BELL) ? 0 : 1;
+    // Nor (NOPF) where both operands stay in the 256 MB last-level cache and the launch runs at the
+    // board's power limit: the extra requests then cost more than the latency they hide
+    // (8192^3: 368.2 -> 364.8 us without, 4096^3: 54.9 -> 53.9 us).
+    constexpr int NPF = (BSTREAM || BELL || NOPF) ? 0 : 1;
     constexpr int pf_dist = 1;
 
     // Start skew: the workgroups of an XCD that work on tile row i of its window start i * skew
@@ -853,7 +857,7 @@ __device__ __forceinline__ void gemm_ptile_body(int M, int K, int N,
     }
 }
 
-template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM>
+template <class S, int AF, int BF, bool KOVER, bool EX, bool BSTREAM, bool NOPF = false>
 __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, int N,
                                                                  const uint8_t *__restrict__ A,
                                                                  const uint8_t *__restrict__ B,
@@ -864,7 +868,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                                                                  int bulk, int tail, int nsplit,
                                                                  int rounds, int rotate_and_skew, OutSpec spec)
 {
-    gemm_ptile_body<S, AF, BF, KOVER, EX, BSTREAM, false>(M, K, N, A, B, C, ws, counters, tiles_m, tiles_n, GM, CB, bulk, tail,
+    gemm_ptile_body<S, AF, BF, KOVER, EX, BSTREAM, false, NOPF>(M, K, N, A, B, C, ws, counters, tiles_m, tiles_n, GM, CB, bulk, tail,
                                                           nsplit, rounds, rotate_and_skew, spec, BellSpec{nullptr, 0, 0, 0});
 }
 
@@ -881,7 +885,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_bell_kernel(int M, int 
                                                                       int rounds, int rotate_and_skew, BellSpec bell)
 {
     const OutSpec plain = {1.0f, nullptr, nullptr, FP8GEMM_DEV_OUT_F32, 0.0f, nullptr, FP8GEMM_DEV_OUT_F32, nullptr, nullptr, nullptr};
-    gemm_ptile_body<S, AF, BF, false, false, false, true>(M, K, N, A, B, C, ws, counters, tiles_m, tiles_n, GM, CB, bulk, tail,
+    gemm_ptile_body<S, AF, BF, false, false, false, true, false>(M, K, N, A, B, C, ws, counters, tiles_m, tiles_n, GM, CB, bulk, tail,
                                                           nsplit, rounds, rotate_and_skew, plain, bell);
 }
 
