@@ -131,11 +131,16 @@ __global__ __launch_bounds__(256) void spmv_bell_kernel(int m, int k, int block,
                                                          const int *__restrict__ block_cols,
                                                          const uint8_t *__restrict__ x, float *__restrict__ y)
 {
-    constexpr int DEPTH = 4;
+    constexpr int DEPTH = 8;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_x[];      // x, then 4 KiB for the waves' sums
     const int xbytes = (k + 15) & ~15;
-    for (int t = threadIdx.x * 16; t < k; t += 256 * 16) *reinterpret_cast<v4i *>(lds_x + t) = load_piece(x + t);
-    __syncthreads();
+    bool x_staged = false;
+    // (x is staged in LDS after the first loads of S have been issued, so that their latencies overlap)
+    auto stage_x = [&]() __attribute__((always_inline)) {
+        for (int t = threadIdx.x * 16; t < k; t += 256 * 16) *reinterpret_cast<v4i *>(lds_x + t) = load_piece(x + t);
+        __syncthreads();
+        x_staged = true;
+    };
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int i = lane & 15, q = lane >> 4;
     const int kell = ell_cols * block;
@@ -172,6 +177,7 @@ __global__ __launch_bounds__(256) void spmv_bell_kernel(int m, int k, int block,
 #pragma unroll
             for (int d = 0; d < DEPTH; ++d)
                 if (d < mine) fetch(d, d);
+            if (!x_staged) stage_x();                                  // (uniform over the workgroup: first pass of every wave)
             for (int u0 = 0; u0 < mine; u0 += DEPTH) {
 #pragma unroll
                 for (int d = 0; d < DEPTH; ++d) {
@@ -185,6 +191,7 @@ __global__ __launch_bounds__(256) void spmv_bell_kernel(int m, int k, int block,
                 }
             }
         }
+        if (!x_staged) stage_x();                                      // a wave without a group still joins the barrier
         if (ksplit > 1) {
             v4f *sums = reinterpret_cast<v4f *>(lds_x + xbytes);
             sums[wave * 64 + lane] = acc;
@@ -198,6 +205,7 @@ __global__ __launch_bounds__(256) void spmv_bell_kernel(int m, int k, int block,
         }
         if (ksplit > 1) break;
     }
+    if (!x_staged) stage_x();          // a wave that had no group at all: every wave passes the barrier exactly once
 }
 
 // y[row] = sum over the stored entries of the row of float(values[e]) * float(x[col[e]]):
@@ -225,7 +233,7 @@ __global__ __launch_bounds__(256) void spmv_csr_kernel(int m, const uint8_t *__r
 }
 
 // The same with 16-byte loads of the indices and 4-byte loads of the values (four entries per lane
-// and pass, two passes in flight), waves that walk a few rows each (row w, w + waves, ..), and x in LDS
+// and pass, four passes in flight), waves that walk a few rows each (row w, w + waves, ..), and x in LDS
 // (XLDS: k <= kSpmvLdsBytes; otherwise x is gathered through the caches).  A row's entries are taken in
 // aligned groups of four starting at the group that holds its first entry; entries of the neighbouring
 // rows in the first and last group are masked out, and the last groups of the arrays are read
@@ -239,16 +247,6 @@ __global__ __launch_bounds__(256) void spmv_csr_vec_kernel(int m, int k, const u
                                                             const uint8_t *__restrict__ x, float *__restrict__ y)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_x[];
-    if (XLDS) {
-        // (k need not be a multiple of 16: the tail goes byte by byte)
-        const int k16 = k & ~15;
-        const bool aligned = reinterpret_cast<uintptr_t>(x) % 16 == 0;
-        if (aligned)
-            for (int t = threadIdx.x * 16; t < k16; t += 256 * 16) *reinterpret_cast<v4i *>(lds_x + t) = load_piece(x + t);
-        for (int t = (aligned ? k16 : 0) + threadIdx.x; t < k; t += 256) lds_x[t] = x[t];
-        __syncthreads();
-    }
-    const uint8_t *xs = XLDS ? lds_x : x;
     const int lane = threadIdx.x & 63;
     const int waves = gridDim.x * 4;
     const int nnz = row_offsets[m];
@@ -260,6 +258,16 @@ __global__ __launch_bounds__(256) void spmv_csr_vec_kernel(int m, int k, const u
         e0 = row_offsets[row];
         e1 = row_offsets[row + 1];
     }
+    if (XLDS) {
+        // (k need not be a multiple of 16: the tail goes byte by byte)
+        const int k16 = k & ~15;
+        const bool aligned = reinterpret_cast<uintptr_t>(x) % 16 == 0;
+        if (aligned)
+            for (int t = threadIdx.x * 16; t < k16; t += 256 * 16) *reinterpret_cast<v4i *>(lds_x + t) = load_piece(x + t);
+        for (int t = (aligned ? k16 : 0) + threadIdx.x; t < k; t += 256) lds_x[t] = x[t];
+        __syncthreads();
+    }
+    const uint8_t *xs = XLDS ? lds_x : x;
     while (w < m) {
         // the next row's bounds are on their way while this row is added up
         const int wn = w + waves;
@@ -286,9 +294,31 @@ __global__ __launch_bounds__(256) void spmv_csr_vec_kernel(int m, int k, const u
                     if (e + t < nnz) one(e + t);
             }
         };
-        for (int e = (e0 & ~3) + lane * 4; e < e1; e += 512) {
-            four(e);
-            if (e + 256 < e1) four(e + 256);
+        for (int e = (e0 & ~3) + lane * 4; e < e1; e += 1024) {
+            // four passes of 256 entries in flight: the loads first, then the arithmetic
+            v4i c4[4];
+            uint32_t v4[4];
+            bool vec[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int eu = e + 256 * u;
+                vec[u] = eu < e1 && eu + 4 <= vec_end;
+                if (vec[u]) {
+                    c4[u] = *reinterpret_cast<const v4i *>(col + eu);
+                    v4[u] = *reinterpret_cast<const uint32_t *>(values + eu);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int eu = e + 256 * u;
+                if (vec[u]) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        if (eu + t >= e0 && eu + t < e1) acc += fp8_to_float<SF>((v4[u] >> (8 * t)) & 0xFFu) * fp8_to_float<XF>(xs[c4[u][t]]);
+                } else if (eu < e1) {
+                    four(eu);                      // the last groups of the arrays, element by element
+                }
+            }
         }
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
