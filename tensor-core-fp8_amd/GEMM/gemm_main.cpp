@@ -13,6 +13,13 @@
 // is an addition: it runs and times only the CPU reference path, without
 // touching the GPU.
 //
+// Kernels 10 to 13 are additions for the sparse kernels the reference's README plans (SpMM, SpMV;
+// README.md:7): 10 SpMM and 11 SpMV with S (dimM x dimK) in blocked-ELL form, 12 SpMM and 13 SpMV
+// with S in compressed sparse rows, e4m3 x e4m3, operands from the generators of
+// include/bm_test_utils.h (GenerateUniformBlockedELLIndex, MakeSparseMatrixRandomUniform,
+// SortedRowSwizzle).  GEMM_SPARSE_BLOCK (default 128) and GEMM_SPARSE_KEEP (share of blocks or
+// elements kept, default 0.25 / 0.1) shape the operand; dimN is the number of dense columns (SpMV: 1).
+//
 // Differences kept on purpose: verification counts its errors (the reference's
 // `if(num_errors = 0)` assigns) and uses the bound
 // |C_gpu - C_ref| <= 2*K*2^-24 * sum_k |a*b| next to the reference's absolute
@@ -272,13 +279,180 @@ void BmFN(int M, int K, int N, int kernel, bool func, bool record, const Options
     std::printf("end BmFN\n");
 }
 
+// ---- sparse kernels ------------------------------------------------------------------
+// CPU reference: out[i][j] = sum over the stored entries of row i, in storage order, of
+// float(value) * float(B[j][column]) -- the loop of cpu_reference_gemm with the zeros left out.
+// S receives sum |a*b| per output.
+template <typename SType, typename BType>
+static void cpu_reference_spmm(int M, int K, int N, const SType *values, const int *row_offsets, const int *col, const BType *B,
+                               float *out, double *S)
+{
+    float lutS[256], lutB[256];
+    for (int c = 0; c < 256; ++c) {
+        lutS[c] = fp8::decode((uint8_t)c, SType::format);
+        lutB[c] = fp8::decode((uint8_t)c, BType::format);
+    }
+#pragma omp parallel for schedule(dynamic, 4)
+    for (int i = 0; i < M; ++i)
+        for (int j = 0; j < N; ++j) {
+            const BType *brow = B + (size_t)j * K;
+            float acc = 0.0f;
+            double sabs = 0.0;
+            for (int e = row_offsets[i]; e < row_offsets[i + 1]; ++e) {
+                const float p = lutS[values[e].x] * lutB[brow[col[e]].x];
+                acc += p;
+                sabs += std::fabs((double)p);
+            }
+            out[(size_t)i * N + j] = acc;
+            S[(size_t)i * N + j] = sabs;
+        }
+}
+
+static double env_number(const char *name, double fallback)
+{
+    const char *v = std::getenv(name);
+    return v ? std::atof(v) : fallback;
+}
+
+// kernel 10: SpMM blocked-ELL, 11: SpMV blocked-ELL, 12: SpMM CSR, 13: SpMV CSR (rows longest first)
+template <typename SType, typename BType>
+static void BmSparse(int M, int K, int N, int kernel, bool func, bool record)
+{
+    const bool bell = kernel == 10 || kernel == 11, vec = kernel == 11 || kernel == 13;
+    if (vec) N = 1;
+    std::default_random_engine generator;
+    std::vector<SType> h_val;
+    std::vector<int> h_off, h_col, h_bcols, h_order;
+    int block = 0, ell = 0;
+    if (bell) {
+        block = (int)env_number("GEMM_SPARSE_BLOCK", 128);
+        if (block <= 0 || block % 16 != 0 || M % block != 0 || K % block != 0) {
+            std::printf("blocked-ELL needs dimM and dimK to be multiples of the block (%d), a multiple of 16\n", block);
+            return;
+        }
+        const int nbr = M / block, nbc = K / block;
+        ell = std::max(1, std::min(nbc, (int)std::lround(nbc * env_number("GEMM_SPARSE_KEEP", 0.25))));
+        h_bcols.resize((size_t)nbr * ell);
+        GenerateUniformBlockedELLIndex(nbc, ell, nbr, h_bcols.data(), generator);
+        h_val.resize((size_t)M * ell * block);
+        MakeDenseMatrix<SType>(M, ell * block, h_val.data(), generator);
+        // the same operand as rows of entries, for the CPU loop
+        h_off.resize(M + 1);
+        h_col.resize(h_val.size());
+        for (int i = 0; i <= M; ++i) h_off[i] = i * ell * block;
+        for (int i = 0; i < M; ++i)
+            for (int t = 0; t < ell * block; ++t) h_col[(size_t)i * ell * block + t] = h_bcols[(size_t)(i / block) * ell + t / block] * block + t % block;
+    } else {
+        const double keep = env_number("GEMM_SPARSE_KEEP", 0.1);
+        const int nonzeros = (int)std::max(1.0, std::min((double)M * K, keep * (double)M * K));
+        const int padding = 4;
+        h_val.resize((size_t)nonzeros + (size_t)M * (padding - 1));
+        h_col.resize(h_val.size());
+        h_off.resize(M + 1);
+        const int64_t stored = MakeSparseMatrixRandomUniform<SType, int>(M, K, nonzeros, h_val.data(), h_off.data(), h_col.data(), generator, padding);
+        h_val.resize(stored);
+        h_col.resize(stored);
+        h_order.resize(M);
+        SortedRowSwizzle(M, h_off.data(), h_order.data());
+    }
+    std::vector<BType> h_B((size_t)N * K);
+    MakeDenseMatrix<BType>(N, K, h_B.data(), generator);
+    const size_t stored = h_val.size();
+    std::printf("%s %s: S %d x %d with %zu stored entries (%.1f %%)%s, %d dense column%s\n", bell ? "blocked-ELL" : "CSR", vec ? "SpMV" : "SpMM", M, K,
+                stored, 100.0 * stored / ((double)M * K), bell ? (" in blocks of " + std::to_string(block)).c_str() : "", N, N == 1 ? "" : "s");
+
+    std::vector<float> h_ref;
+    std::vector<double> h_scale;
+    if (func) {
+        h_ref.assign((size_t)M * N, 0.0f);
+        h_scale.assign((size_t)M * N, 0.0);
+        cpu_reference_spmm(M, K, N, h_val.data(), h_off.data(), h_col.data(), h_B.data(), h_ref.data(), h_scale.data());
+    }
+    SType *d_val;
+    BType *d_B;
+    float *d_C;
+    int *d_off = nullptr, *d_col = nullptr, *d_bcols = nullptr, *d_order = nullptr;
+    checkHip(hipMalloc(&d_val, stored * sizeof(SType)));
+    checkHip(hipMalloc(&d_B, h_B.size() * sizeof(BType)));
+    checkHip(hipMalloc(&d_C, (size_t)M * N * sizeof(float)));
+    checkHip(hipMemcpy(d_val, h_val.data(), stored * sizeof(SType), hipMemcpyHostToDevice));
+    checkHip(hipMemcpy(d_B, h_B.data(), h_B.size() * sizeof(BType), hipMemcpyHostToDevice));
+    auto upload = [](const std::vector<int> &h, int **d) {
+        checkHip(hipMalloc(d, h.size() * sizeof(int)));
+        checkHip(hipMemcpy(*d, h.data(), h.size() * sizeof(int), hipMemcpyHostToDevice));
+    };
+    if (bell) {
+        upload(h_bcols, &d_bcols);
+    } else {
+        upload(h_off, &d_off);
+        upload(h_col, &d_col);
+        upload(h_order, &d_order);
+    }
+    const int fs = SType::format, fb = BType::format;
+    auto launch = [&]() -> hipError_t {
+        int code;
+        if (kernel == 10) code = fp8gemm_spmm_bell(M, K, N, block, ell, d_val, fs, d_bcols, d_B, fb, d_C, nullptr);
+        else if (kernel == 11) code = fp8gemm_spmv_bell(M, K, block, ell, d_val, fs, d_bcols, d_B, fb, d_C, nullptr);
+        else if (kernel == 12) code = fp8gemm_spmm_csr(M, K, N, d_val, fs, d_off, d_col, d_B, fb, d_C, nullptr);
+        else code = fp8gemm_spmv_csr(M, K, d_val, fs, d_off, d_col, d_order, d_B, fb, d_C, nullptr);
+        return static_cast<hipError_t>(code);
+    };
+    hipEvent_t start, end;
+    checkHip(hipEventCreate(&start));
+    checkHip(hipEventCreate(&end));
+    for (int i = 0; i < warmup; ++i) checkHip(launch());
+    float batch_msec = 0.0f;
+    checkHip(hipEventRecord(start));
+    for (int i = 0; i < repeat; ++i) checkHip(launch());
+    checkHip(hipEventRecord(end));
+    checkHip(hipEventSynchronize(end));
+    checkHip(hipEventElapsedTime(&batch_msec, start, end));
+    const double usec = batch_msec / repeat * 1e3;
+    const double flop = 2.0 * (double)stored * N;
+    const double bytes = (double)stored * (bell ? 1.0 : 5.0) + (double)N * K + 4.0 * (double)M * N;
+    const double gflops = flop / usec / 1e3, gbs = bytes / usec / 1e3;
+    std::printf("batch of %d launches: %.3f us per launch, %.1f GFlops on the stored entries, %.1f GB/s (%.1f%% of %.0f)\n", repeat, usec,
+                gflops, gbs, gbs / kPeakHbmGBs * 100.0, kPeakHbmGBs);
+    if (record) record_csv(kernel, M, K, N, gflops, usec, gbs);
+    if (func) {
+        std::vector<float> h_C((size_t)M * N);
+        checkHip(hipMemcpy(h_C.data(), d_C, h_C.size() * sizeof(float), hipMemcpyDeviceToHost));
+        size_t num_errors = 0;
+        double max_error = 0.0, worst_ratio = 0.0;
+        for (size_t i = 0; i < h_C.size(); ++i) {
+            const double err = std::fabs((double)h_C[i] - (double)h_ref[i]);
+            // reordered fp32 sums over at most K terms, plus what the MFMA's groups of 8 products can drop (2^-13 of
+            // eight times the largest product of a group, bounded by 2^-10 of the sum of magnitudes)
+            const double tol = (2.0 * K * std::ldexp(1.0, -24) + std::ldexp(1.0, -10)) * h_scale[i];
+            if (!(err <= tol)) ++num_errors;
+            if (err > max_error) max_error = err;
+            if (tol > 0 && err / tol > worst_ratio) worst_ratio = err / tol;
+        }
+        if (num_errors == 0)
+            std::printf("Result Verified!\n");
+        else
+            std::cout << "There are " << num_errors << " errors." << std::endl;
+        std::printf("MAx Error is %f\n", max_error);
+        std::printf("worst |err| / tolerance = %.4g\n", worst_ratio);
+    }
+    checkHip(hipEventDestroy(start));
+    checkHip(hipEventDestroy(end));
+    checkHip(hipFree(d_val));
+    checkHip(hipFree(d_B));
+    checkHip(hipFree(d_C));
+    for (int *p : {d_off, d_col, d_bcols, d_order})
+        if (p) checkHip(hipFree(p));
+    std::printf("end BmSparse\n");
+}
+
 static void usage(void)
 {
     std::printf("!!!!!!!\n");
     std::printf("Input Help!\n");
     std::printf("Input Format is  ./gemm_main [dimM] [dimK] [dimN] [kernel] [verify] [reocrd] [testbench] [dist [seed]]\n");
     std::printf("dim: M-K-N in GEMM\n");
-    std::printf("kernel: {1,2: e4m3*e4m3  3,4: e5m2*e5m2  5,6: e4m3*e5m2  7,8: e5m2*e4m3; odd = 2-stage, even = 4-stage; 0: CPU path only}\n");
+    std::printf("kernel: {1,2: e4m3*e4m3  3,4: e5m2*e5m2  5,6: e4m3*e5m2  7,8: e5m2*e4m3; odd = 2-stage, even = 4-stage; 0: CPU path only;\n");
+    std::printf("         10: SpMM blocked-ELL  11: SpMV blocked-ELL  12: SpMM CSR  13: SpMV CSR}\n");
     std::printf("verify: {0 not verify result with cpu, 1: verify result}\n");
     std::printf("record: {record in csv files}\n");
     std::printf("testbench: {1: sweep square sizes 256..16384}\n");
@@ -308,6 +482,10 @@ static bool run_kernel(int kernel, int M, int K, int N, bool verify, bool record
     case 7: case 8:
         std::printf("e5m2 * e4m3 = fp32\n");
         BmFN<e5m2, e4m3, float>(M, K, N, kernel, verify, record, opt);
+        return true;
+    case 10: case 11: case 12: case 13:
+        std::printf("sparse e4m3 * e4m3 = fp32\n");
+        BmSparse<e4m3, e4m3>(M, K, N, kernel, verify, record);
         return true;
     default:
         std::printf("unsupported kernel\n");

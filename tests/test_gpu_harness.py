@@ -137,3 +137,27 @@ def test_vendor_comparator_runs_both_libraries_and_compares_them(pkg, tmp_path):
     check(run(5, 256, 512, 256), [(256, 256, 256), (512, 512, 512)])
     check(run(5, "shape", 16, 1024, 512), [(16, 512, 1024)])
     assert subprocess.run([exe], capture_output=True, text=True).returncode == 1      # usage
+
+
+@pytest.mark.parametrize("kernel,shape,env", [
+    (10, (512, 1024, 300), {}),                                     # blocked-ELL SpMM, 128 x 128 blocks: the tiled kernel
+    (10, (512, 1024, 300), {"GEMM_SPARSE_BLOCK": "256", "GEMM_SPARSE_KEEP": "0.5"}),
+    (10, (256, 512, 40), {"GEMM_SPARSE_BLOCK": "32"}),               # small blocks: the direct kernel
+    (11, (2048, 4096, 1), {"GEMM_SPARSE_BLOCK": "64"}),              # blocked-ELL SpMV
+    (12, (300, 1024, 200), {}),                                      # CSR SpMM through the dense scratch
+    (13, (3000, 2048, 1), {"GEMM_SPARSE_KEEP": "0.05"}),             # CSR SpMV, longest rows first
+])
+def test_sparse_kernel_ids(harness, kernel, shape, env):
+    """Kernel ids 10..13: the sparse kernels on operands from the re-created generators of the
+    reference's bm_test_utils.h (blocked-ELL column lists, CSR with row padding, sorted row
+    order), timed and verified against the harness's own CPU loop over the stored entries."""
+    M, K, N = shape
+    r = harness(M, K, N, kernel, 1, 0, 0, env=env)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    assert "sparse e4m3 * e4m3 = fp32" in r.stdout
+    assert "Result Verified!" in r.stdout and "errors." not in r.stdout, r.stdout[-1500:]
+    m = re.search(r"worst \|err\| / tolerance = ([0-9.eE+-]+)", r.stdout)
+    assert m and float(m.group(1)) < 1.0
+    g = re.search(r"([0-9.]+) GFlops on the stored entries", r.stdout)
+    assert g and float(g.group(1)) > 0.0
+    assert "end BmSparse" in r.stdout
