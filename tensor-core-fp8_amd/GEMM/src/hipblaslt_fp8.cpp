@@ -5,8 +5,10 @@
 // Stands where the reference's cuBLASLt sample stands (GEMM/src/cublas.cu with
 // the TestBench of GEMM/include/helper.h): same problem set-up (op(A) = T with
 // lda = k, op(B) = N with ldb = k, i.e. A row-major m x k and B stored n x k, the
-// operand layout of gemm::GEMM), per-tensor scale pointers for A and B (fp32 C and D
-// take none here), a 32 MiB workspace, the first heuristic result, `repeat` launches timed one by
+// operand layout of gemm::GEMM), per-tensor scale pointers for A and B (and, in `sample`
+// mode, for C and D and the pointer that receives the largest |D|, as cublas.cu:41-46 hands
+// them over; dropped again, with a note, if the library offers no algorithm with them for an
+// fp32 D), a 32 MiB workspace, the first heuristic result, `repeat` launches timed one by
 // one with events and averaged (cublas.cu:66-94; here after a warm-up and in blocks that
 // alternate between the two libraries, so that both see the same clocks), and a sweep over
 // 256, 512, .. 16384 (cublas.cu:123-130).
@@ -17,7 +19,9 @@
 //    the matrix pipe depends on the data;
 //  * alpha = 1, beta = 0 and unit scales by default, so that the call computes
 //    what gemm::GEMM computes and the two results can be compared; the
-//    sample's alpha = 2, beta = 1, scales 2 / 0.5 are available as `sample`;
+//    sample's alpha = 2, beta = 1, scales 2 / 0.5 / 1 / 1 are available as `sample`, where
+//    this library's side is fp8gemm_launch_epilogue with the same scalars and pointers and the
+//    two results (and largest magnitudes) are compared as well;
 //  * the rate is printed in true GFLOP/s (2mnk / seconds / 1e9); the sample
 //    divides by 1024 * 1024 and milliseconds (cublas.cu:101).
 //
@@ -60,7 +64,7 @@ struct Problem {
     size_t workspace_bytes;
     void *a = nullptr, *b = nullptr, *workspace = nullptr;
     float *c = nullptr, *d = nullptr, *ours = nullptr;
-    float *scales = nullptr;   // device: a_scale, b_scale
+    float *scales = nullptr;   // device: a_scale, b_scale, c_scale, d_scale, amax of the vendor's D, amax of ours
 
     Problem(int m_, int n_, int k_, float alpha_, float beta_, float a_scale, float b_scale, size_t ws)
         : m(m_), n(n_), k(k_), alpha(alpha_), beta(beta_), workspace_bytes(ws)
@@ -74,11 +78,11 @@ struct Problem {
         check_hip(hipMalloc(&d, (size_t)m * n * sizeof(float)), "hipMalloc D");
         check_hip(hipMalloc(&ours, (size_t)m * n * sizeof(float)), "hipMalloc ours");
         check_hip(hipMalloc(&workspace, workspace_bytes), "hipMalloc workspace");
-        check_hip(hipMalloc(&scales, 2 * sizeof(float)), "hipMalloc scales");
+        check_hip(hipMalloc(&scales, 6 * sizeof(float)), "hipMalloc scales");
         check_hip(hipMemcpy(a, ha.data(), ha.size(), hipMemcpyHostToDevice), "copy A");
         check_hip(hipMemcpy(b, hb.data(), hb.size(), hipMemcpyHostToDevice), "copy B");
         check_hip(hipMemset(c, 0, (size_t)m * n * sizeof(float)), "clear C");
-        const float hs[2] = {a_scale, b_scale};
+        const float hs[6] = {a_scale, b_scale, 1.0f, 1.0f, -1.0f, -1.0f};      // C and D scales as in the sample (helper.h:62)
         check_hip(hipMemcpy(scales, hs, sizeof(hs), hipMemcpyHostToDevice), "copy scales");
     }
     ~Problem()
@@ -163,7 +167,26 @@ bool run_size(hipblasLtHandle_t handle, Problem &p, int repeat, bool comparable)
              "workspace");
     hipblasLtMatmulHeuristicResult_t heur = {};
     int found = 0;
-    check_lt(hipblasLtMatmulAlgoGetHeuristic(handle, op, la, lb, lc, ld, pref, 1, &heur, &found), "heuristic");
+    bool vendor_amax = false;
+    if (!comparable) {
+        // the sample also hands over scale pointers for C and D and a pointer for the largest |D|
+        const float *sc = p.scales + 2, *sd = p.scales + 3;
+        float *amax = p.scales + 4;
+        const bool set = hipblasLtMatmulDescSetAttribute(op, HIPBLASLT_MATMUL_DESC_C_SCALE_POINTER, &sc, sizeof(sc)) == HIPBLAS_STATUS_SUCCESS &&
+                         hipblasLtMatmulDescSetAttribute(op, HIPBLASLT_MATMUL_DESC_D_SCALE_POINTER, &sd, sizeof(sd)) == HIPBLAS_STATUS_SUCCESS &&
+                         hipblasLtMatmulDescSetAttribute(op, HIPBLASLT_MATMUL_DESC_AMAX_D_POINTER, &amax, sizeof(amax)) == HIPBLAS_STATUS_SUCCESS;
+        if (set && hipblasLtMatmulAlgoGetHeuristic(handle, op, la, lb, lc, ld, pref, 1, &heur, &found) == HIPBLAS_STATUS_SUCCESS && found > 0) {
+            vendor_amax = true;
+        } else {
+            printf("(no hipBLASLt algorithm takes C / D scale and amax pointers for an fp32 D: A and B scales only)\n");
+            const void *none = nullptr;
+            (void)hipblasLtMatmulDescSetAttribute(op, HIPBLASLT_MATMUL_DESC_C_SCALE_POINTER, &none, sizeof(none));
+            (void)hipblasLtMatmulDescSetAttribute(op, HIPBLASLT_MATMUL_DESC_D_SCALE_POINTER, &none, sizeof(none));
+            (void)hipblasLtMatmulDescSetAttribute(op, HIPBLASLT_MATMUL_DESC_AMAX_D_POINTER, &none, sizeof(none));
+            found = 0;
+        }
+    }
+    if (found == 0) check_lt(hipblasLtMatmulAlgoGetHeuristic(handle, op, la, lb, lc, ld, pref, 1, &heur, &found), "heuristic");
     bool ok = found > 0;
     if (!ok) {
         printf("no heuristic function available for current configuration\n");
@@ -174,10 +197,16 @@ bool run_size(hipblasLtHandle_t handle, Problem &p, int repeat, bool comparable)
                      "matmul");
         };
         auto own = [&] {
-            const int e = fp8gemm_launch(p.m, p.k, p.n, p.a, FP8GEMM_E4M3, p.b, FP8GEMM_E4M3, p.ours, 2, nullptr);
+            // the plain launch, or (sample mode) the epilogue entry point with the sample's scalars and pointers;
+            // C holds zeros, so its layout (column-major there, row-major here) does not matter
+            const int e = comparable
+                              ? fp8gemm_launch(p.m, p.k, p.n, p.a, FP8GEMM_E4M3, p.b, FP8GEMM_E4M3, p.ours, 2, nullptr)
+                              : fp8gemm_launch_epilogue(p.m, p.k, p.n, p.a, FP8GEMM_E4M3, p.b, FP8GEMM_E4M3, p.ours, FP8GEMM_OUT_F32, p.alpha,
+                                                        p.beta, p.c, FP8GEMM_OUT_F32, p.scales, p.scales + 1, p.scales + 2, p.scales + 3,
+                                                        p.scales + 5, nullptr);
             if (e != 0) {
-                printf("fp8gemm_launch failed: %d %s\n", e, fp8gemm_error_string(e));
-                throw std::runtime_error("fp8gemm_launch failed");
+                printf("fp8gemm launch failed: %d %s\n", e, fp8gemm_error_string(e));
+                throw std::runtime_error("fp8gemm launch failed");
             }
         };
         vendor();
@@ -191,7 +220,7 @@ bool run_size(hipblasLtHandle_t handle, Problem &p, int repeat, bool comparable)
                flop / (ms_vendor * 1e-3) / 1e9);
         printf("GEMM-fp8gemm-fp8:   M[%d] x N[%d] x K[%d], performance = %lfGFLOPS (%f ms).\n", p.m, p.n, p.k,
                flop / (ms_own * 1e-3) / 1e9, ms_own);
-        if (comparable) {
+        {
             // D is column-major m x n, ours row-major m x n: D[i + j*m] against ours[i*n + j]
             // on a strided sample; both are fp32 sums of the same products in different orders
             std::vector<float> hd((size_t)p.m * p.n), ho((size_t)p.m * p.n);
@@ -207,6 +236,14 @@ bool run_size(hipblasLtHandle_t handle, Problem &p, int repeat, bool comparable)
             }
             printf("max |hipblaslt - fp8gemm| = %g (largest |C| = %g, sqrt(K) * 2^-24 * that = %g)\n", worst, scale,
                    std::sqrt((double)p.k) * std::ldexp(1.0, -24) * scale);
+            if (!comparable) {
+                float amax[2] = {0.0f, 0.0f};
+                check_hip(hipMemcpy(amax, p.scales + 4, sizeof(amax), hipMemcpyDeviceToHost), "copy amax");
+                if (vendor_amax)
+                    printf("largest |D|: hipblaslt %g, fp8gemm %g\n", amax[0], amax[1]);
+                else
+                    printf("largest |D|: fp8gemm %g (hipblaslt took no amax pointer)\n", amax[1]);
+            }
         }
     }
     if (pref) check_lt(hipblasLtMatmulPreferenceDestroy(pref), "destroy");

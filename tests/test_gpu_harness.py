@@ -136,6 +136,16 @@ def test_vendor_comparator_runs_both_libraries_and_compares_them(pkg, tmp_path):
 
     check(run(5, 256, 512, 256), [(256, 256, 256), (512, 512, 512)])
     check(run(5, "shape", 16, 1024, 512), [(16, 512, 1024)])
+    # the reference sample's scalars and pointers (alpha 2, beta 1, scales 2 / 0.5 / 1 / 1, amax): this library's
+    # side is the epilogue entry point, and the two results and largest magnitudes are compared
+    out = run(5, 256, 512, 256, "sample")
+    check(out, [(256, 256, 256), (512, 512, 512)])
+    both = re.findall(r"largest \|D\|: hipblaslt ([0-9.eE+-]+), fp8gemm ([0-9.eE+-]+)", out)
+    own = re.findall(r"largest \|D\|: fp8gemm ([0-9.eE+-]+) \(hipblaslt took no amax pointer\)", out)
+    assert len(both) + len(own) == 2
+    for v, o in both:
+        assert abs(float(v) - float(o)) <= 1e-3 * float(o)
+    assert all(float(o) > 0 for o in own)
     assert subprocess.run([exe], capture_output=True, text=True).returncode == 1      # usage
 
 
