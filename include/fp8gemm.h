@@ -88,8 +88,10 @@ int fp8gemm_gemv(int n, int k, const void *w, int w_fmt, const void *x, int x_fm
  * k % block == 0); every block row stores ell_cols blocks.  values: m x (ell_cols * block)
  * codes row-major, 16-byte aligned (stored block t of a row's block row occupies bytes
  * t * block .. of the row); block_cols: (m / block) x ell_cols ints, the block column of each
- * stored block, or -1 for a padding block that contributes nothing.  The kernel feeds the MFMA
- * from the stored blocks directly; blocks that are not stored cost nothing.  b 16-byte aligned.
+ * stored block, or -1 for a padding block that contributes nothing.  The kernels feed the MFMA
+ * from the stored blocks directly; blocks that are not stored cost nothing.  Blocks of 32 rows and
+ * multiples run on the LDS-tiled kernel of the GEMM (n >= 64), other sizes on a kernel without
+ * LDS.  b 16-byte aligned.
  */
 int fp8gemm_spmm_bell(int m, int k, int n, int block, int ell_cols, const void *values, int s_fmt, const int *block_cols,
                       const void *b, int b_fmt, float *out, void *stream);

@@ -96,12 +96,13 @@ struct OutSpec {
 // A sparse A in blocked-ELL form for the tiled kernel (kernel_sparse.h describes the format): A
 // is then the m x K matrix of stored values (K = ell_cols * block bytes per row), and K tile g of a
 // tile row pairs with the bytes of B's rows at block column cols[tile row's block row][g * BK / block].
-// block % BK == 0 and block % BM == 0, so a K tile lies inside one stored block and all rows of a
-// tile share one list.
+// block % BM == 0, so all rows of a tile share one list; with block % BK == 0 a K tile lies inside
+// one stored block, with smaller blocks it spans several (`sub`).
 struct BellSpec {
     const int *cols;      // (m / block) x ell_cols block column numbers, -1 = padding (counts as zeros)
     int ell_cols, block;
     int kb;               // row stride of B in bytes (the k of the sparse matrix)
+    int sub;              // blocks smaller than a K tile: gcd(block, 128), the bytes of a K tile that share a stored block
 };
 
 __device__ __forceinline__ float out_scale(const OutSpec &o)

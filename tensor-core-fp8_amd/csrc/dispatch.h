@@ -30,6 +30,10 @@ using TileT2 = TileShape<192, 256, 128, 2, 2, 2, 3>;  // three-quarter-height ti
 using TileE5 = TileShape<64, 128, 128, 1, 4, 5, 3>;    // up to 64 rows of A: four waves of 64 x 32, 5 x 24 KiB ring
 using TileQ4s = TileShape<128, 128, 128, 2, 2, 4, 3>;  // up to 128 rows: the quarter tile with a 4 x 32 KiB ring
 
+// blocked-ELL operands with blocks of 64 and 32 rows: tiles as tall as a block, four waves side by side
+using TileB64 = TileShape<64, 256, 128, 1, 4, 3, 3>;   // 64 x 64 per wave, 3 x 40 KiB ring
+using TileB32 = TileShape<32, 256, 128, 1, 4, 4, 3>;   // 32 x 64 per wave, 4 x 36 KiB ring
+
 // Skinny kernel shapes: <MT, TN, BK, stages>.
 template <int MT, int TN>
 using SkinnyV0 = SkinnyShape<MT, TN, 128, 5>;
@@ -204,8 +208,9 @@ template <class S, int AF, int BF>
 hipError_t launch_ptile_bell(int m, int kell, int n, const uint8_t *values, const uint8_t *b, float *out, const BellSpec &bell,
                              int nsplit, bool split_all, int rotate, Workspace &wsp, hipStream_t stream)
 {
-    if (bell.block % S::BM != 0 || bell.block % S::BK != 0 || kell % S::BK != 0 || kell > (1 << 23) || bell.kb > (1 << 23) ||
-        nsplit < 1 || nsplit > kell / S::BK)
+    const bool small = S::BM < 128;              // blocks below a K tile: any stored row length, sub-blocks of 32 bytes or more
+    if (bell.block % S::BM != 0 || (small ? bell.sub < 32 : (bell.block % S::BK != 0 || kell % S::BK != 0)) || kell % 16 != 0 ||
+        kell > (1 << 23) || bell.kb > (1 << 23) || nsplit < 1 || nsplit > (kell + S::BK - 1) / S::BK)
         return hipErrorInvalidValue;
     const PtileWork w = ptile_work(m, n, S::BM, S::BN, nsplit, split_all);
     if (!w.ok) return hipErrorInvalidValue;
@@ -239,6 +244,20 @@ template <int AF, int BF>
 hipError_t dispatch_bell(int m, int kell, int n, const uint8_t *values, const uint8_t *b, float *out, const BellSpec &bell,
                          Workspace &wsp, hipStream_t stream)
 {
+    if (bell.block % 128 != 0) {
+        // small blocks: tiles as tall as a block; too few tiles for the chip are cut into K slices
+        const int bm = bell.block % 64 == 0 ? 64 : 32;
+        const long tiles = (long)(m / bm) * ((n + 255) / 256);
+        const int kt = (kell + 127) / 128;
+        int nsplit = 1;
+        if (tiles < 256) {
+            nsplit = (int)((256 + tiles - 1) / tiles);
+            if (nsplit > kt / 8) nsplit = kt / 8;
+            if (nsplit < 1) nsplit = 1;
+        }
+        if (bm == 64) return launch_ptile_bell<TileB64, AF, BF>(m, kell, n, values, b, out, bell, nsplit, nsplit > 1, 2, wsp, stream);
+        return launch_ptile_bell<TileB32, AF, BF>(m, kell, n, values, b, out, bell, nsplit, nsplit > 1, 2, wsp, stream);
+    }
     // tile shapes whose rows share one block row: 128-row tiles, and 256-row ones where the blocks are that tall
     unsigned allowed = (1u << 5) | (1u << 6);
     if (bell.block % 256 == 0) allowed |= (1u << 0) | (1u << 13);

@@ -503,9 +503,10 @@ hipError_t launch_spmv_bell(int m, int k, int block, int ell_cols, const uint8_t
 
 bool fmt_ok(int f) { return f == FP8GEMM_E4M3 || f == FP8GEMM_E5M2; }
 
-// the tiled kernel's tiles are 128 rows or more and its K tiles 128 bytes; below 64 columns of
-// output a 128-column tile is mostly empty
-bool bell_tiled(int block, int n) { return block % 128 == 0 && n >= 64; }
+// The tiled kernel takes blocks whose rows fill whole tiles (32, 64, 128 or 256 rows: block % 32 == 0)
+// and whose bytes inside a 128-byte K tile come in runs of 32 or more (the same condition); below 64
+// columns of output its tiles are mostly empty.
+bool bell_tiled(int block, int n) { return block % 32 == 0 && n >= 64; }
 
 }  // namespace
 
@@ -536,11 +537,13 @@ int fp8gemm_spmm_bell(int m, int k, int n, int block, int ell_cols, const void *
     hipStream_t s = static_cast<hipStream_t>(stream);
     (void)hipGetLastError();
     hipError_t e;
-    // Blocks that hold whole 128-byte K tiles and whole 128-row tiles go through the LDS-tiled
-    // persistent kernel (the stored values are its A, the block list steers where the K tiles of
-    // B come from); other block sizes, and outputs of a few columns, through the direct kernel.
+    // Blocks of 32 rows and multiples go through the LDS-tiled persistent kernel (the stored values
+    // are its A, the block list steers where the K tiles of B, or with blocks below 128 the parts of
+    // a K tile, come from); other block sizes, and outputs of a few columns, through the direct kernel.
     if (bell_tiled(block, n)) {
-        const BellSpec bell = {block_cols, ell_cols, block, k};
+        int sub = 128;                                  // gcd(block, 128)
+        while (block % sub != 0) sub /= 2;
+        const BellSpec bell = {block_cols, ell_cols, block, k, sub};
         const int kell = ell_cols * block;
         Workspace wsp = Workspace::pooled(s);
         if (s_fmt == FP8GEMM_E4M3 && b_fmt == FP8GEMM_E4M3)

@@ -133,7 +133,12 @@ __device__ __forceinline__ void gemm_ptile_body(int M, int K, int N,
                                                 int bulk, int tail, int nsplit,
                                                 int rounds, int rotate_and_skew, OutSpec spec, BellSpec bell)
 {
-    static_assert(!BELL || (!KOVER && !BSTREAM), "the blocked-ELL form has whole K tiles and shares B between tile rows");
+    static_assert(!BELL || !BSTREAM, "the blocked-ELL form shares B between tile rows");
+    // Small blocks (tiles of fewer than 128 rows): a 128-byte K tile spans several stored blocks, so
+    // where a chunk of B lies depends on which `bell.sub` bytes of the K tile (one stored block, or the
+    // part of one) it belongs to; the offsets then ride in the loads' per-lane offsets.
+    constexpr bool BELL_SMALL = BELL && S::BM < 128;
+    constexpr int BELL_SUBS = BELL_SMALL ? 4 : 1;  // sub-blocks of a K tile at most (bell.sub >= 32)
     const int KB = BELL ? bell.kb : K;             // row stride of B
     const int rotate = rotate_and_skew & 0xFF;
     const int skew = rotate_and_skew >> 8;
@@ -241,7 +246,12 @@ __device__ __forceinline__ void gemm_ptile_body(int M, int K, int N,
         const int per = j < S::A_LOADS ? S::A_LOADS : S::B_LOADS;
         const int row = (wave * per + jj) * RPI + lrow;
         ld_off[j] = (uint32_t)row * (uint32_t)(j < S::A_LOADS ? K : KB) + (uint32_t)((lslot ^ tile_swizzle<BK, S::SWZ>(row)) * 16);
+        // (small blocks: B's chunk counts from the start of its sub-block, whose place the block list gives)
+        if (BELL_SMALL && j >= S::A_LOADS) ld_off[j] -= (uint32_t)((((lslot ^ tile_swizzle<BK, S::SWZ>(row)) * 16) / bell.sub) * bell.sub);
     }
+    // which sub-block of a K tile this lane's chunks of B lie in: the swizzle only ever changes the
+    // lowest bit of the chunk number between a lane's loads, and a sub-block holds two chunks or more
+    const int bell_sb = BELL_SMALL ? ((lslot ^ tile_swizzle<BK, S::SWZ>(lrow)) * 16) / bell.sub : 0;
     const uint32_t ldsA = lds_base + (uint32_t)(wave * S::A_LOADS * RPI * BK);
     const uint32_t ldsB = lds_base + (uint32_t)(BM * BK + wave * S::B_LOADS * RPI * BK);
     v4i rsA = {0, 0, 0, 0}, rsB = {0, 0, 0, 0};
@@ -285,22 +295,32 @@ __device__ __forceinline__ void gemm_ptile_body(int M, int K, int N,
     // holds that byte offset for walk step 64 * bell_chunk + l (-1: a padding block), so the K loop
     // gets it with v_readlane_b32 and no memory access; a fresh set of 64 is fetched when the walk
     // crosses into the next chunk (a vector load whose wait drains the ring once per 64 K tiles).
+    // Small blocks: one such register per sub-block of a K tile, and bell_vat = the offset of this
+    // lane's sub-block in the K tile being loaded.
     const int *bell_row = nullptr;                 // block column list of the planned item's block row
-    int bell_at = -1, bell_chunk = -1;
+    int bell_at[BELL_SUBS], bell_chunk = -1;
+#pragma unroll
+    for (int u = 0; u < BELL_SUBS; ++u) bell_at[u] = -1;
     uint32_t bell_koff = 0;                        // ... of the K tile being loaded
     bool bell_pad = false;                         // ... or that it is a padding block
+    int bell_vat = -1;
     auto bell_fetch = [&](int chunk) __attribute__((always_inline)) {
         const int tt = chunk * 64 + lane;
-        int v = -1;
-        if (tt < kt_count) {
-            int kk = tt + kt_rot;
-            kk = kk >= kt_count ? kk - kt_count : kk;
-            const int pos = (kt_base + kk) * BK;                    // byte position in the stored row
-            const int blk = pos / bell.block;
-            const int c = bell_row[blk];
-            v = c < 0 ? -1 : c * bell.block + (pos - blk * bell.block);
+#pragma unroll
+        for (int u = 0; u < BELL_SUBS; ++u) {
+            int v = -1;
+            if (tt < kt_count && (!BELL_SMALL || u * bell.sub < BK)) {
+                int kk = tt + kt_rot;
+                kk = kk >= kt_count ? kk - kt_count : kk;
+                const int pos = (kt_base + kk) * BK + (BELL_SMALL ? u * bell.sub : 0);   // byte position in the stored row
+                if (pos < K) {                                          // (small blocks: the last K tile may overhang the stored row)
+                    const int blk = pos / bell.block;
+                    const int c = bell_row[blk];
+                    v = c < 0 ? -1 : c * bell.block + (pos - blk * bell.block);
+                }
+            }
+            bell_at[u] = v;
         }
-        bell_at = v;
         bell_chunk = chunk;
     };
     auto plan_loads = [&](int tile_m, int tile_n, int kt0, int count, int item) __attribute__((always_inline)) {
@@ -339,9 +359,25 @@ __device__ __forceinline__ void gemm_ptile_body(int M, int K, int N,
         if constexpr (BELL) {
             if (j == S::A_LOADS) {                 // first load of B of this K tile: where its block lies
                 if ((ktile >> 6) != bell_chunk) bell_fetch(ktile >> 6);               // (uniform, once per 64 K tiles)
-                const int at = __builtin_amdgcn_readlane(bell_at, ktile & 63);
-                bell_pad = at < 0;
-                bell_koff = (uint32_t)at;
+                if constexpr (BELL_SMALL) {
+                    int mine = __builtin_amdgcn_readlane(bell_at[0], ktile & 63);
+#pragma unroll
+                    for (int u = 1; u < BELL_SUBS; ++u) {
+                        const int at = __builtin_amdgcn_readlane(bell_at[u], ktile & 63);
+                        mine = bell_sb == u ? at : mine;
+                    }
+                    bell_vat = mine;
+                } else {
+                    const int at = __builtin_amdgcn_readlane(bell_at[0], ktile & 63);
+                    bell_pad = at < 0;
+                    bell_koff = (uint32_t)at;
+                }
+            }
+            if (BELL_SMALL && j >= S::A_LOADS) {
+                // (a padding block, or past the end of the stored row: outside the extent, reads zeros)
+                buffer_load_lds_b128(rsB, ldsB + sbase + (uint32_t)((j - S::A_LOADS) * RPI * BK),
+                                     bell_vat < 0 ? 0xFFFFFFF0u : ld_off[j] + (uint32_t)bell_vat, 0u);
+                return;
             }
             if (j >= S::A_LOADS) {
                 // a padding block: every lane's address goes outside the extent and reads zeros
@@ -869,7 +905,7 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_kernel(int M, int K, in
                                                                  int rounds, int rotate_and_skew, OutSpec spec)
 {
     gemm_ptile_body<S, AF, BF, KOVER, EX, BSTREAM, false, NOPF>(M, K, N, A, B, C, ws, counters, tiles_m, tiles_n, GM, CB, bulk, tail,
-                                                          nsplit, rounds, rotate_and_skew, spec, BellSpec{nullptr, 0, 0, 0});
+                                                          nsplit, rounds, rotate_and_skew, spec, BellSpec{nullptr, 0, 0, 0, 0});
 }
 
 // The same kernel with A in blocked-ELL form: out = S * B^T, S stored as `A` (M x K values) and `bell`.
@@ -885,7 +921,8 @@ __global__ __launch_bounds__(S::THREADS) void gemm_ptile_bell_kernel(int M, int 
                                                                       int rounds, int rotate_and_skew, BellSpec bell)
 {
     const OutSpec plain = {1.0f, nullptr, nullptr, FP8GEMM_DEV_OUT_F32, 0.0f, nullptr, FP8GEMM_DEV_OUT_F32, nullptr, nullptr, nullptr};
-    gemm_ptile_body<S, AF, BF, false, false, false, true, false>(M, K, N, A, B, C, ws, counters, tiles_m, tiles_n, GM, CB, bulk, tail,
+    // (tiles of fewer than 128 rows serve small blocks, whose stored rows need not be whole K tiles)
+    gemm_ptile_body<S, AF, BF, (S::BM < 128), false, false, true, false>(M, K, N, A, B, C, ws, counters, tiles_m, tiles_n, GM, CB, bulk, tail,
                                                           nsplit, rounds, rotate_and_skew, plain, bell);
 }
 

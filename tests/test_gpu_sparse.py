@@ -85,7 +85,27 @@ def test_spmm_bell_through_the_tiled_kernel(pkg, oracle, fs, fb, block, ell, m, 
 
 
 @pytest.mark.parametrize("fs,fb", PAIRS)
-@pytest.mark.parametrize("block", [128, 256])
+@pytest.mark.parametrize("block,ell,m,k,n", [(64, 40, 128, 4096, 300), (96, 3, 192, 960, 128), (192, 2, 384, 1536, 256),
+                                              (32, 9, 2048, 1024, 2048), (32, 1, 32, 32, 64), (64, 3, 4096, 512, 1100),
+                                              (160, 5, 320, 1600, 70)])
+def test_spmm_bell_small_blocks_through_the_tiled_kernel(pkg, oracle, fs, fb, block, ell, m, k, n):
+    """Blocks of 32 rows and multiples that are not multiples of 128 run on the tiled kernel with
+    tiles as tall as a block (64 or 32 rows): a K tile then spans several stored blocks (or parts
+    of blocks: 96, 160, 192), stored rows need not be whole K tiles, few tiles are cut into K
+    slices, many run in rounds with leftover tiles; padding blocks everywhere."""
+    rng = np.random.default_rng(zlib.crc32(repr(("small", fs, fb, block, ell, m, k, n)).encode()))
+    vals, bcols = random_bell(rng, m, k, block, ell, fs, pad_some=ell > 1)
+    B = random_codes(rng, (n, k), fb)
+    if fb == 1:
+        B = np.where(((B >> 2) & 0x1F) > 24, B & 0x83 | 0x3C, B).astype(np.uint8)
+    out = pkg.spmm_bell(dev(vals), dev(bcols), block, dev(B), k, s_fmt=fs, b_fmt=fb).cpu().numpy()
+    v, offs, col = oracle.bell_to_csr(vals, bcols, block)
+    ref, tol = bound(oracle, v, fs, offs, col, k, B, fb, mfma=True)
+    check(out, ref, tol)
+
+
+@pytest.mark.parametrize("fs,fb", PAIRS)
+@pytest.mark.parametrize("block", [32, 64, 128, 256])
 def test_spmm_bell_tiled_one_hot_is_bit_exact(pkg, oracle, fs, fb, block):
     """The tiled kernel's gather through the block list, bit for bit: one value of 1.0 per row of S."""
     one = {0: 0x38, 1: 0x3C}
