@@ -19,18 +19,30 @@
 
 #include "device_common.h"
 
-// fp8 code -> float, by the bits (exact; subnormals, infinities and NaNs included)
+// fp8 code (the lowest byte of `code`) -> float through the conversion instructions, which on gfx950
+// take the OCP formats: exact for every code, subnormals, infinities and NaNs included (held to that by
+// the one-hot tests: a row with a single 1.0 must return the other operand's decoded value bit for bit).
 template <int F>
 __device__ __forceinline__ float fp8_to_float(uint32_t code)
 {
-    if (F == 1) {      // E5M2 is the upper byte of an IEEE half
-        return (float)__builtin_bit_cast(_Float16, (unsigned short)(code << 8));
+    return F == 1 ? __builtin_amdgcn_cvt_f32_bf8((int)code, 0) : __builtin_amdgcn_cvt_f32_fp8((int)code, 0);
+}
+
+// the four codes of a 32-bit word
+template <int F>
+__device__ __forceinline__ void fp8x4_to_float(uint32_t w, float out[4])
+{
+    if (F == 1) {
+        out[0] = __builtin_amdgcn_cvt_f32_bf8((int)w, 0);
+        out[1] = __builtin_amdgcn_cvt_f32_bf8((int)w, 1);
+        out[2] = __builtin_amdgcn_cvt_f32_bf8((int)w, 2);
+        out[3] = __builtin_amdgcn_cvt_f32_bf8((int)w, 3);
+    } else {
+        out[0] = __builtin_amdgcn_cvt_f32_fp8((int)w, 0);
+        out[1] = __builtin_amdgcn_cvt_f32_fp8((int)w, 1);
+        out[2] = __builtin_amdgcn_cvt_f32_fp8((int)w, 2);
+        out[3] = __builtin_amdgcn_cvt_f32_fp8((int)w, 3);
     }
-    const uint32_t sign = (code & 0x80u) << 24;
-    const uint32_t e = (code >> 3) & 0xFu, mant = code & 7u;
-    if ((code & 0x7Fu) == 0x7Fu) return __builtin_bit_cast(float, sign | 0x7FC00000u);
-    if (e == 0) return __builtin_bit_cast(float, sign | __builtin_bit_cast(uint32_t, (float)mant * 0.001953125f));   // mant * 2^-9
-    return __builtin_bit_cast(float, sign | ((e + 120u) << 23) | (mant << 20));
 }
 
 __device__ __forceinline__ v4i load_piece(const uint8_t *p)
@@ -286,8 +298,11 @@ __global__ __launch_bounds__(256) void spmv_csr_vec_kernel(int m, int k, const u
                 const v4i c4 = *reinterpret_cast<const v4i *>(col + e);
                 const uint32_t v4 = *reinterpret_cast<const uint32_t *>(values + e);
 #pragma unroll
+                float v[4];
+                fp8x4_to_float<SF>(v4, v);
+#pragma unroll
                 for (int t = 0; t < 4; ++t)
-                    if (e + t >= e0 && e + t < e1) acc += fp8_to_float<SF>((v4 >> (8 * t)) & 0xFFu) * fp8_to_float<XF>(xs[c4[t]]);
+                    if (e + t >= e0 && e + t < e1) acc += v[t] * fp8_to_float<XF>(xs[c4[t]]);
             } else {
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
@@ -312,9 +327,11 @@ __global__ __launch_bounds__(256) void spmv_csr_vec_kernel(int m, int k, const u
             for (int u = 0; u < 4; ++u) {
                 const int eu = e + 256 * u;
                 if (vec[u]) {
+                    float v[4];
+                    fp8x4_to_float<SF>(v4[u], v);
 #pragma unroll
                     for (int t = 0; t < 4; ++t)
-                        if (eu + t >= e0 && eu + t < e1) acc += fp8_to_float<SF>((v4[u] >> (8 * t)) & 0xFFu) * fp8_to_float<XF>(xs[c4[u][t]]);
+                        if (eu + t >= e0 && eu + t < e1) acc += v[t] * fp8_to_float<XF>(xs[c4[u][t]]);
                 } else if (eu < e1) {
                     four(eu);                      // the last groups of the arrays, element by element
                 }

@@ -188,6 +188,28 @@ def test_spmv_csr(pkg, oracle, fs, fx, m, k, density, pad):
     assert np.array_equal(y2, y)          # the order of the rows changes no row's sum
 
 
+@pytest.mark.parametrize("fs,fx", PAIRS)
+def test_spmv_csr_decodes_every_code_bit_for_bit(pkg, oracle, fs, fx):
+    """One stored entry per row: a value of 1.0 against every code of x's format, and every code of the
+    value's format against an x of 1.0 -- the kernel's own decode (conversion instructions) must give
+    the oracle's value bit for bit, subnormals, -0 and the infinities of e5m2 included; NaN codes give NaN."""
+    one = {0: 0x38, 1: 0x3C}
+    k = 256
+    codes = np.arange(256, dtype=np.uint8)
+    offs = np.arange(257, dtype=np.int32)
+    col = np.arange(256, dtype=np.int32)
+    for vals, x, decoded in [(np.full(256, one[fs], np.uint8), codes, oracle.decode(codes, fx)),
+                             (codes, np.full(256, one[fx], np.uint8), oracle.decode(codes, fs))]:
+        want = oracle.spmm_csr(vals, fs, offs, col, k, x, fx)          # = the decoded values (a sum that starts at +0 turns -0 into +0)
+        assert np.array_equal(np.nan_to_num(want, nan=7.0), np.nan_to_num(decoded + np.float32(0.0), nan=7.0))
+        for aligned in (True, False):                      # the 16-byte-load kernel and the element-wise one
+            dcol = dev(np.concatenate([[0], col]).astype(np.int32))[1:] if not aligned else dev(col)
+            y = pkg.spmm_csr(dev(vals), dev(offs), dcol, dev(x), k, s_fmt=fs, b_fmt=fx).cpu().numpy()
+            nan = np.isnan(want)
+            assert np.array_equal(np.isnan(y), nan)
+            assert np.array_equal(y[~nan].view(np.uint32), want[~nan].view(np.uint32))
+
+
 def test_spmv_csr_small_integers_with_duplicates_exact(pkg, oracle):
     """|values| <= 8: every sum is an exact integer; entries that repeat a column are added."""
     rng = np.random.default_rng(3)
