@@ -495,6 +495,23 @@ def main():
                        "us": ms3 * 1e3, "dense_equivalent_tflops": 2.0 * m3 * k3 * n3 / ms3 / 1e9,
                        "note": "S is written out as a dense fp8 matrix in scratch, then the dense GEMM runs"})
         del v, o, c, Bd, Cd, xv, yv
+        # sampled dense-dense product: 8192 x 8192 outputs in column vectors of 8, one vector in ten kept, K = 512
+        m_vec, vec, n4, k4 = 1024, 8, 8192, 512
+        mask = rng.random((m_vec, n4)) < 0.10
+        offs = np.concatenate([[0], np.cumsum(mask.sum(axis=1))]).astype(np.int32)
+        colh = np.nonzero(mask)[1].astype(np.int32)
+        nnz = int(offs[-1])
+        o, c = torch.from_numpy(offs).to(dev), torch.from_numpy(colh).to(dev)
+        Ld = torch.from_numpy(pkg.fill((m_vec * vec, k4), pkg.E4M3, seed=0x5BA + 11, dist="normal")).to(dev)
+        Rd = torch.from_numpy(pkg.fill((n4, k4), pkg.E4M3, seed=0x5BA + 12, dist="normal")).to(dev)
+        Od = torch.empty((nnz, vec), dtype=torch.float32, device=dev)
+        ms4 = raw_time(lambda i: ck(L.fp8gemm_sddmm(m_vec, k4, vec, o.data_ptr(), c.data_ptr(), Ld.data_ptr(), 0, Rd.data_ptr(), 0,
+                                                    Od.data_ptr(), stream)), 60)
+        sparse.append({"kernel": "fp8gemm_sddmm", "rows": m_vec * vec, "cols": n4, "K": k4, "vec_length": vec, "stored_vectors": nnz,
+                       "density": nnz / (m_vec * n4), "us": ms4 * 1e3, "tflops_on_stored_outputs": 2.0 * nnz * vec * k4 / ms4 / 1e9,
+                       "gathered_rhs_gbs": nnz * k4 / ms4 / 1e6,
+                       "note": "every stored vector reads one row of rhs (K bytes) out of cache; vec_length 8 fills half of the MFMA's rows"})
+        del o, c, Ld, Rd, Od
         torch.cuda.empty_cache()
 
     # ---------------------------------------------------------------- CPU baseline (host cores)

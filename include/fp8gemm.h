@@ -74,7 +74,7 @@ int fp8gemm_launch(int m, int k, int n, const void *a, int a_fmt, const void *b,
 int fp8gemm_gemv(int n, int k, const void *w, int w_fmt, const void *x, int x_fmt, float *y, void *stream);
 
 /*
- * ---- Sparse operands: SpMM and SpMV ---------------------------------------------------
+ * ---- Sparse operands: SpMM, SpMV and SDDMM ---------------------------------------------
  * out = S * B^T with S (m x k) sparse and B dense, stored n x k like the B of the GEMM; out is
  * m x n fp32 row-major, overwritten; n = 1 with a vector x of k codes is the SpMV.  The
  * reference names SpMM and SpMV as planned kernels (README.md:7) and holds none; what it holds
@@ -114,6 +114,17 @@ int fp8gemm_spmv_csr(int m, int k, const void *values, int s_fmt, const int *row
 int fp8gemm_spmm_csr(int m, int k, int n, const void *values, int s_fmt, const int *row_offsets, const int *col_idx,
                      const void *b, int b_fmt, float *out, void *stream);
 size_t fp8gemm_spmm_csr_scratch_bytes(int m, int k, int n);
+/*
+ * Sampled dense-dense product with a vector-sparse output pattern, the loop of the reference's host
+ * helper Host_sddmm (GEMM/include/bm_test_utils.h:172-194):
+ *     out[j * vec_length + v] = sum_l float(lhs[(i * vec_length + v) * k + l]) * float(rhs[col_idx[j] * k + l])
+ * for every vector row i < m_vec, every stored entry j in [row_offsets[i], row_offsets[i+1]) and every
+ * v < vec_length.  lhs: (m_vec * vec_length) x k, rhs: n x k, both row-major codes (col_idx < n); out:
+ * row_offsets[m_vec] x vec_length floats.  All device pointers.  vec_length <= 16 with k % 16 == 0 and
+ * 16-byte aligned operands runs on the MFMA; anything else one thread per output.
+ */
+int fp8gemm_sddmm(int m_vec, int k, int vec_length, const int *row_offsets, const int *col_idx, const void *lhs, int l_fmt,
+                  const void *rhs, int r_fmt, float *out, void *stream);
 /*
  * Host helper: rows ordered by falling number of stored entries (ties in rising row number),
  * the order of the reference's SortedRowSwizzle (GEMM/include/bm_test_utils.h:202-216).

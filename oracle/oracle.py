@@ -56,6 +56,8 @@ def lib():
                                                         i32p, ctypes.c_int, f32p, f64p]
     L.oracle_spmm_csr.restype = None
     L.oracle_spmm_csr.argtypes = [ctypes.c_int] * 3 + [u8p, ctypes.c_int, i32p, i32p, u8p, ctypes.c_int, f32p, f64p]
+    L.oracle_sddmm.restype = None
+    L.oracle_sddmm.argtypes = [ctypes.c_int] * 3 + [i32p, i32p, u8p, ctypes.c_int, u8p, ctypes.c_int, f32p, f64p]
     L.oracle_num_threads.restype = ctypes.c_int
     L.oracle_set_num_threads.argtypes = [ctypes.c_int]
     _lib = L
@@ -137,6 +139,24 @@ def spmm_csr(values, sfmt, row_offsets, col, k, B, bfmt, with_scale=False):
     if vector:
         out = out[:, 0]
         S = S[:, 0] if with_scale else None
+    return (out, S) if with_scale else out
+
+
+def sddmm(row_offsets, col, vec, lhs, lfmt, rhs, rfmt, with_scale=False):
+    """Sampled dense-dense product (the reference's Host_sddmm, GEMM/include/bm_test_utils.h:172-194):
+    out[j*vec + v] = lhs[i*vec + v] . rhs[col[j]] for every stored entry j of vector row i.
+    lhs: (m_vec*vec, k) codes, rhs: (n, k) codes.  Returns (nnz, vec) fp32."""
+    row_offsets = np.ascontiguousarray(row_offsets, dtype=np.int32)
+    col = np.ascontiguousarray(col, dtype=np.int32)
+    lhs = np.ascontiguousarray(lhs, dtype=np.uint8)
+    rhs = np.ascontiguousarray(rhs, dtype=np.uint8)
+    m_vec, k = row_offsets.size - 1, lhs.shape[1]
+    assert lhs.shape[0] == m_vec * vec and rhs.shape[1] == k and row_offsets[-1] == col.size
+    assert col.size == 0 or (col.min() >= 0 and col.max() < rhs.shape[0])
+    out = np.empty((col.size, vec), dtype=np.float32)
+    S = np.empty((col.size, vec), dtype=np.float64) if with_scale else None
+    lib().oracle_sddmm(m_vec, k, vec, _p(row_offsets, ctypes.c_int), _p(col, ctypes.c_int), _p(lhs, ctypes.c_uint8), lfmt,
+                       _p(rhs, ctypes.c_uint8), rfmt, _p(out, ctypes.c_float), _p(S, ctypes.c_double) if with_scale else None)
     return (out, S) if with_scale else out
 
 

@@ -445,6 +445,98 @@ static void BmSparse(int M, int K, int N, int kernel, bool func, bool record)
     std::printf("end BmSparse\n");
 }
 
+// kernel 14: sampled dense-dense product, dimM x dimN outputs in column vectors of GEMM_SDDMM_VEC (8) rows, the
+// fraction GEMM_SPARSE_KEEP (0.1) of the vectors stored, at uniformly drawn places
+template <typename LType, typename RType>
+static void BmSddmm(int M, int K, int N, bool func, bool record)
+{
+    const int vec = (int)env_number("GEMM_SDDMM_VEC", 8);
+    if (vec <= 0 || M % vec != 0) {
+        std::printf("SDDMM needs dimM to be a multiple of the vector length (%d)\n", vec);
+        return;
+    }
+    const int m_vec = M / vec;
+    std::default_random_engine generator;
+    const double keep = env_number("GEMM_SPARSE_KEEP", 0.1);
+    const int vectors = (int)std::max(1.0, std::min((double)m_vec * N, keep * (double)m_vec * N));
+    std::vector<LType> unused(vectors);
+    std::vector<int> h_off(m_vec + 1), h_col(vectors);
+    const int64_t stored = MakeSparseMatrixRandomUniform<LType, int>(m_vec, N, vectors, unused.data(), h_off.data(), h_col.data(), generator, 0);
+    std::vector<LType> h_L((size_t)M * K);
+    std::vector<RType> h_R((size_t)N * K);
+    MakeDenseMatrix<LType>(M, K, h_L.data(), generator);
+    MakeDenseMatrix<RType>(N, K, h_R.data(), generator);
+    std::printf("SDDMM: %d x %d outputs in vectors of %d, %lld vectors stored (%.1f %%), K = %d\n", M, N, vec, (long long)stored,
+                100.0 * stored / ((double)m_vec * N), K);
+    LType *d_L;
+    RType *d_R;
+    float *d_out;
+    int *d_off, *d_col;
+    checkHip(hipMalloc(&d_L, h_L.size()));
+    checkHip(hipMalloc(&d_R, h_R.size()));
+    checkHip(hipMalloc(&d_out, (size_t)stored * vec * sizeof(float)));
+    checkHip(hipMalloc(&d_off, h_off.size() * sizeof(int)));
+    checkHip(hipMalloc(&d_col, h_col.size() * sizeof(int)));
+    checkHip(hipMemcpy(d_L, h_L.data(), h_L.size(), hipMemcpyHostToDevice));
+    checkHip(hipMemcpy(d_R, h_R.data(), h_R.size(), hipMemcpyHostToDevice));
+    checkHip(hipMemcpy(d_off, h_off.data(), h_off.size() * sizeof(int), hipMemcpyHostToDevice));
+    checkHip(hipMemcpy(d_col, h_col.data(), h_col.size() * sizeof(int), hipMemcpyHostToDevice));
+    auto launch = [&]() -> hipError_t {
+        return static_cast<hipError_t>(fp8gemm_sddmm(m_vec, K, vec, d_off, d_col, d_L, LType::format, d_R, RType::format, d_out, nullptr));
+    };
+    hipEvent_t start, end;
+    checkHip(hipEventCreate(&start));
+    checkHip(hipEventCreate(&end));
+    for (int i = 0; i < warmup; ++i) checkHip(launch());
+    float batch_msec = 0.0f;
+    checkHip(hipEventRecord(start));
+    for (int i = 0; i < repeat; ++i) checkHip(launch());
+    checkHip(hipEventRecord(end));
+    checkHip(hipEventSynchronize(end));
+    checkHip(hipEventElapsedTime(&batch_msec, start, end));
+    const double usec = batch_msec / repeat * 1e3;
+    const double gflops = 2.0 * (double)stored * vec * K / usec / 1e3;
+    const double gbs = ((double)stored * K + (double)M * K + 4.0 * (double)stored * (vec + 1)) / usec / 1e3;
+    std::printf("batch of %d launches: %.3f us per launch, %.1f GFlops on the stored outputs, %.1f GB/s of gathered rows and results\n", repeat,
+                usec, gflops, gbs);
+    if (record) record_csv(14, M, K, N, gflops, usec, gbs);
+    if (func) {
+        std::vector<float> h_out((size_t)stored * vec), h_ref((size_t)stored * vec);
+        checkHip(hipMemcpy(h_out.data(), d_out, h_out.size() * sizeof(float), hipMemcpyDeviceToHost));
+        Host_sddmm<LType, float>(m_vec, K, vec, h_off.data(), h_col.data(), h_L.data(), h_R.data(), h_ref.data());
+        size_t num_errors = 0;
+        double max_error = 0.0, worst_ratio = 0.0;
+        for (int i = 0; i < m_vec; ++i)
+            for (int j = h_off[i]; j < h_off[i + 1]; ++j)
+                for (int v = 0; v < vec; ++v) {
+                    double sabs = 0.0;
+                    const LType *l = h_L.data() + ((size_t)i * vec + v) * K;
+                    const RType *r = h_R.data() + (size_t)h_col[j] * K;
+                    for (int t = 0; t < K; ++t) sabs += std::fabs((double)float(l[t]) * (double)float(r[t]));
+                    const size_t at = (size_t)j * vec + v;
+                    const double err = std::fabs((double)h_out[at] - (double)h_ref[at]);
+                    const double tol = (2.0 * K * std::ldexp(1.0, -24) + std::ldexp(1.0, -10)) * sabs;
+                    if (!(err <= tol)) ++num_errors;
+                    if (err > max_error) max_error = err;
+                    if (tol > 0 && err / tol > worst_ratio) worst_ratio = err / tol;
+                }
+        if (num_errors == 0)
+            std::printf("Result Verified!\n");
+        else
+            std::cout << "There are " << num_errors << " errors." << std::endl;
+        std::printf("MAx Error is %f\n", max_error);
+        std::printf("worst |err| / tolerance = %.4g\n", worst_ratio);
+    }
+    checkHip(hipEventDestroy(start));
+    checkHip(hipEventDestroy(end));
+    checkHip(hipFree(d_L));
+    checkHip(hipFree(d_R));
+    checkHip(hipFree(d_out));
+    checkHip(hipFree(d_off));
+    checkHip(hipFree(d_col));
+    std::printf("end BmSddmm\n");
+}
+
 static void usage(void)
 {
     std::printf("!!!!!!!\n");
@@ -452,7 +544,7 @@ static void usage(void)
     std::printf("Input Format is  ./gemm_main [dimM] [dimK] [dimN] [kernel] [verify] [reocrd] [testbench] [dist [seed]]\n");
     std::printf("dim: M-K-N in GEMM\n");
     std::printf("kernel: {1,2: e4m3*e4m3  3,4: e5m2*e5m2  5,6: e4m3*e5m2  7,8: e5m2*e4m3; odd = 2-stage, even = 4-stage; 0: CPU path only;\n");
-    std::printf("         10: SpMM blocked-ELL  11: SpMV blocked-ELL  12: SpMM CSR  13: SpMV CSR}\n");
+    std::printf("         10: SpMM blocked-ELL  11: SpMV blocked-ELL  12: SpMM CSR  13: SpMV CSR  14: SDDMM}\n");
     std::printf("verify: {0 not verify result with cpu, 1: verify result}\n");
     std::printf("record: {record in csv files}\n");
     std::printf("testbench: {1: sweep square sizes 256..16384}\n");
@@ -486,6 +578,10 @@ static bool run_kernel(int kernel, int M, int K, int N, bool verify, bool record
     case 10: case 11: case 12: case 13:
         std::printf("sparse e4m3 * e4m3 = fp32\n");
         BmSparse<e4m3, e4m3>(M, K, N, kernel, verify, record);
+        return true;
+    case 14:
+        std::printf("sampled e4m3 * e4m3 = fp32\n");
+        BmSddmm<e4m3, e4m3>(M, K, N, verify, record);
         return true;
     default:
         std::printf("unsupported kernel\n");

@@ -131,4 +131,25 @@ inline void SortedRowSwizzle(int rows, const int *row_offsets, int *row_indices)
     });
 }
 
+// Host loop of the sampled dense-dense product (the reference's Host_sddmm,
+// GEMM/include/bm_test_utils.h:172-194): the output pattern has m_vec rows of column vectors of
+// VecLength; stored vector j of row i receives, for v < VecLength, the running fp32 sum along K of
+// lhs_matrix[i * VecLength + v][:] * rhs_matrix[col_indices[j]][:], both operands row-major with k
+// columns.  output_values: row_offsets[m_vec] x VecLength.
+template <typename ValueType, typename OutType>
+void Host_sddmm(int m_vec, int k, int VecLength, const int *row_offsets, const int *col_indices, const ValueType *lhs_matrix,
+                const ValueType *rhs_matrix, OutType *output_values)
+{
+    for (int i = 0; i < m_vec; ++i)
+        for (int j = row_offsets[i]; j < row_offsets[i + 1]; ++j) {
+            const ValueType *right = rhs_matrix + static_cast<size_t>(col_indices[j]) * k;
+            for (int v = 0; v < VecLength; ++v) {
+                const ValueType *left = lhs_matrix + (static_cast<size_t>(i) * VecLength + v) * k;
+                float sum = 0.0f;
+                for (int l = 0; l < k; ++l) sum += static_cast<float>(left[l]) * static_cast<float>(right[l]);
+                output_values[static_cast<size_t>(j) * VecLength + v] = static_cast<OutType>(sum);
+            }
+        }
+}
+
 #endif  // BM_TEST_UTILS_H

@@ -126,6 +126,8 @@ def lib():
     L.fp8gemm_spmm_csr.argtypes = [ci, ci, ci, vp, ci, ip, ip, vp, ci, vp, vp]
     L.fp8gemm_spmm_csr_scratch_bytes.restype = ctypes.c_size_t
     L.fp8gemm_spmm_csr_scratch_bytes.argtypes = [ci, ci, ci]
+    L.fp8gemm_sddmm.restype = ci
+    L.fp8gemm_sddmm.argtypes = [ci, ci, ci, ip, ip, vp, ci, vp, ci, vp, vp]
     L.fp8gemm_sorted_row_swizzle.restype = None
     L.fp8gemm_sorted_row_swizzle.argtypes = [ci, ip, ip]
     _lib = L
@@ -373,4 +375,19 @@ def sorted_row_swizzle(row_offsets):
     row_offsets = np.ascontiguousarray(row_offsets, dtype=np.int32)
     out = np.empty(row_offsets.size - 1, dtype=np.int32)
     lib().fp8gemm_sorted_row_swizzle(out.size, row_offsets.ctypes.data, out.ctypes.data)
+    return out
+
+
+def sddmm(row_offsets, col_idx, vec_length, lhs, rhs, l_fmt=None, r_fmt=None, out=None, stream=None):
+    """out[j, v] = lhs[i*vec_length + v] . rhs[col_idx[j]] for every stored entry j of vector row i
+    (row_offsets, col_idx int32 device tensors; lhs (m_vec*vec_length, k), rhs (n, k) codes)."""
+    import torch
+    m_vec = row_offsets.numel() - 1
+    k = lhs.shape[1]
+    if lhs.shape[0] != m_vec * vec_length or rhs.shape[1] != k:
+        raise Fp8GemmError("lhs / rhs do not fit the pattern")
+    if out is None:
+        out = torch.empty((col_idx.numel(), vec_length), dtype=torch.float32, device=lhs.device)
+    check(lib().fp8gemm_sddmm(m_vec, k, vec_length, _dev_ints(row_offsets), _dev_ints(col_idx), lhs.data_ptr(), _fmt_of(lhs, l_fmt),
+                              rhs.data_ptr(), _fmt_of(rhs, r_fmt), out.data_ptr(), _stream_handle(stream)))
     return out

@@ -501,6 +501,24 @@ hipError_t launch_spmv_bell(int m, int k, int block, int ell_cols, const uint8_t
     return hipGetLastError();
 }
 
+template <int LF, int RF>
+hipError_t launch_sddmm(int m_vec, int k, int vec, const int *row_offsets, const int *col, const uint8_t *lhs, const uint8_t *rhs,
+                        float *out, hipStream_t stream)
+{
+    const bool fast = vec <= 16 && k % 16 == 0 && (reinterpret_cast<uintptr_t>(lhs) | reinterpret_cast<uintptr_t>(rhs)) % 16 == 0;
+    const size_t lds = (size_t)vec * (k + kSddmmLdsPad);
+    if (fast && lds <= (size_t)kSddmmLdsBytes)
+        hipLaunchKernelGGL((sddmm_kernel<LF, RF, true>), dim3((unsigned)m_vec), dim3(256), lds, stream, k, vec, row_offsets, col, lhs,
+                           rhs, out);
+    else if (fast)
+        hipLaunchKernelGGL((sddmm_kernel<LF, RF, false>), dim3((unsigned)m_vec), dim3(256), 0, stream, k, vec, row_offsets, col, lhs,
+                           rhs, out);
+    else
+        hipLaunchKernelGGL((sddmm_general_kernel<LF, RF>), dim3((unsigned)m_vec), dim3(256), 0, stream, m_vec, k, vec, row_offsets, col,
+                           lhs, rhs, out);
+    return hipGetLastError();
+}
+
 bool fmt_ok(int f) { return f == FP8GEMM_E4M3 || f == FP8GEMM_E5M2; }
 
 // The tiled kernel takes blocks whose rows fill whole tiles (32, 64, 128 or 256 rows: block % 32 == 0)
@@ -602,6 +620,26 @@ int fp8gemm_spmv_csr(int m, int k, const void *values, int s_fmt, const int *row
         e = launch_spmv_csr<0, 1>(m, k, pv, row_offsets, col_idx, row_order, px, y, s);
     else
         e = launch_spmv_csr<1, 0>(m, k, pv, row_offsets, col_idx, row_order, px, y, s);
+    return (int)e;
+}
+
+int fp8gemm_sddmm(int m_vec, int k, int vec_length, const int *row_offsets, const int *col_idx, const void *lhs, int l_fmt,
+                  const void *rhs, int r_fmt, float *out, void *stream)
+{
+    if (m_vec <= 0 || k <= 0 || vec_length <= 0 || !row_offsets || !col_idx || !lhs || !rhs || !out) return (int)hipErrorInvalidValue;
+    if (!fmt_ok(l_fmt) || !fmt_ok(r_fmt)) return (int)hipErrorInvalidValue;
+    const uint8_t *pl = static_cast<const uint8_t *>(lhs), *pr = static_cast<const uint8_t *>(rhs);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    (void)hipGetLastError();
+    hipError_t e;
+    if (l_fmt == FP8GEMM_E4M3 && r_fmt == FP8GEMM_E4M3)
+        e = launch_sddmm<0, 0>(m_vec, k, vec_length, row_offsets, col_idx, pl, pr, out, s);
+    else if (l_fmt == FP8GEMM_E5M2 && r_fmt == FP8GEMM_E5M2)
+        e = launch_sddmm<1, 1>(m_vec, k, vec_length, row_offsets, col_idx, pl, pr, out, s);
+    else if (l_fmt == FP8GEMM_E4M3)
+        e = launch_sddmm<0, 1>(m_vec, k, vec_length, row_offsets, col_idx, pl, pr, out, s);
+    else
+        e = launch_sddmm<1, 0>(m_vec, k, vec_length, row_offsets, col_idx, pl, pr, out, s);
     return (int)e;
 }
 

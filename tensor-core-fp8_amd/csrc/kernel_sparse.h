@@ -14,6 +14,7 @@
 //     HBM-bound), the matrix-matrix product scatters S into a dense fp8 matrix
 //     (csr_densify_kernel) that the dense GEMM then multiplies: with B stored n x k, an
 //     element-wise kernel would gather single bytes of B at stride k, m * n * nnz_row of them.
+// Also here: the sampled dense-dense product (sddmm_kernel), whose output is sparse instead.
 #ifndef FP8GEMM_KERNEL_SPARSE_H
 #define FP8GEMM_KERNEL_SPARSE_H
 
@@ -297,7 +298,6 @@ __global__ __launch_bounds__(256) void spmv_csr_vec_kernel(int m, int k, const u
             if (e + 4 <= vec_end) {
                 const v4i c4 = *reinterpret_cast<const v4i *>(col + e);
                 const uint32_t v4 = *reinterpret_cast<const uint32_t *>(values + e);
-#pragma unroll
                 float v[4];
                 fp8x4_to_float<SF>(v4, v);
 #pragma unroll
@@ -393,6 +393,104 @@ __global__ __launch_bounds__(256) void csr_densify_rows_kernel(int m, int k, con
         for (int t = threadIdx.x * 16; t < k; t += 256 * 16)
             *reinterpret_cast<v4i *>(dense + (size_t)row * k + t) = *reinterpret_cast<const v4i *>(lds_row + t);
         __syncthreads();
+    }
+}
+
+// Sampled dense-dense product with a vector-sparse output pattern (the reference's Host_sddmm,
+// GEMM/include/bm_test_utils.h:172-194): out[j * vec + v] = lhs[i * vec + v] . rhs[col[j]] for every
+// stored entry j of vector row i; lhs (m_vec * vec) x k and rhs n x k, both row-major: every dot
+// product runs along K on both sides, which is the MFMA's operand layout.  One workgroup of four waves per
+// vector row; a wave takes 16 stored entries at a time (wave, wave + 4, ..): the up to 16 rows of lhs are the
+// MFMA's A, the 16 gathered rows of rhs its B, and out[j][v] is element (v, j) of the 16 x 16 result.
+// Lane (i = lane % 16, q = lane / 16) supplies 32 bytes of row i per K step; the next step's loads are
+// issued before the current MFMA.  The gathered rows of rhs come out of cache at whatever rate the CU can
+// keep loads in flight, so the rows of lhs, which every chunk of the vector row needs again, are taken from
+// LDS instead when they fit (ALDS: rows kSddmmLdsPad bytes apart from a multiple of 128, so that the 16 lanes
+// of a quarter read 16 different bank groups); otherwise they are loaded next to the rows of rhs.
+// Requirements checked by the host: vec <= 16, k % 16 == 0, 16-byte aligned lhs and rhs; ALDS:
+// 16 * (k + kSddmmLdsPad) bytes of dynamic LDS.
+constexpr int kSddmmLdsPad = 16;
+constexpr int kSddmmLdsBytes = 64 * 1024;
+
+template <int LF, int RF, bool ALDS>
+__global__ __launch_bounds__(256) void sddmm_kernel(int k, int vec, const int *__restrict__ row_offsets,
+                                                     const int *__restrict__ col, const uint8_t *__restrict__ lhs,
+                                                     const uint8_t *__restrict__ rhs, float *__restrict__ out)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t sddmm_lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = lane & 15, q = lane >> 4;
+    const int vrow = blockIdx.x;
+    const int e0 = row_offsets[vrow], e1 = row_offsets[vrow + 1];
+    if (e0 >= e1) return;                                     // (the whole workgroup)
+    const int steps = (k + 127) / 128;
+    const v4i zero = {0, 0, 0, 0};
+    // rows of lhs past vec re-read the last one; their results are never stored
+    const int ai = i < vec ? i : vec - 1;
+    const uint8_t *arow = lhs + (size_t)(vrow * vec + ai) * k;
+    const int lds_stride = k + kSddmmLdsPad;
+    if constexpr (ALDS) {
+        const int per_row = k / 16;
+        for (int t = threadIdx.x; t < vec * per_row; t += 256) {
+            const int r = t / per_row, c = t - r * per_row;
+            *reinterpret_cast<v4i *>(sddmm_lds + r * lds_stride + c * 16) = load_piece(lhs + (size_t)(vrow * vec + r) * k + c * 16);
+        }
+        __syncthreads();
+    }
+    const uint8_t *alds = sddmm_lds + ai * lds_stride;
+    for (int j0 = e0 + wave * 16; j0 < e1; j0 += 64) {
+        const int j = j0 + i < e1 ? j0 + i : e1 - 1;          // (entries past the row's end re-read its last one)
+        const uint8_t *brow = rhs + (size_t)col[j] * k;
+        struct Step {
+            v4i a[2], b[2];
+        };
+        auto fetch = [&](int s, Step &f) __attribute__((always_inline)) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int p = s * 128 + (2 * q + h) * 16;
+                if constexpr (!ALDS) f.a[h] = p < k ? load_piece(arow + p) : zero;
+                f.b[h] = p < k ? load_piece(brow + p) : zero;
+            }
+        };
+        v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        Step cur, nxt;
+        fetch(0, cur);
+        for (int s = 0; s < steps; ++s) {
+            if (s + 1 < steps) fetch(s + 1, nxt);
+            if constexpr (ALDS) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int p = s * 128 + (2 * q + h) * 16;
+                    cur.a[h] = p < k ? *reinterpret_cast<const v4i *>(alds + p) : zero;
+                }
+            }
+            acc = mfma_16x16x128<LF, RF>(pack8(cur.a[0], cur.a[1]), pack8(cur.b[0], cur.b[1]), acc);
+            cur = nxt;
+        }
+        // register r of lane (i, q) holds lhs row 4q + r times rhs row col[j0 + i]
+        if (j0 + i < e1) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (4 * q + r < vec) out[(size_t)(j0 + i) * vec + 4 * q + r] = acc[r];
+        }
+    }
+}
+
+// The same for any k, vec and alignment: one thread per output, a running fp32 sum along K.
+template <int LF, int RF>
+__global__ __launch_bounds__(256) void sddmm_general_kernel(int m_vec, int k, int vec, const int *__restrict__ row_offsets,
+                                                             const int *__restrict__ col, const uint8_t *__restrict__ lhs,
+                                                             const uint8_t *__restrict__ rhs, float *__restrict__ out)
+{
+    const int vrow = blockIdx.x;
+    if (vrow >= m_vec) return;
+    const int e0 = row_offsets[vrow], e1 = row_offsets[vrow + 1];
+    for (long t = threadIdx.x; t < (long)(e1 - e0) * vec; t += 256) {
+        const int j = e0 + (int)(t / vec), v = (int)(t % vec);
+        const uint8_t *a = lhs + (size_t)(vrow * vec + v) * k, *b = rhs + (size_t)col[j] * k;
+        float acc = 0.0f;
+        for (int l = 0; l < k; ++l) acc += fp8_to_float<LF>(a[l]) * fp8_to_float<RF>(b[l]);
+        out[(size_t)j * vec + v] = acc;
     }
 }
 

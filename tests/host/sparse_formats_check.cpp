@@ -1,7 +1,8 @@
 // Host check of the sparse operand generators and row orders of the harness
 // (tensor-core-fp8_amd/GEMM/include/bm_test_utils.h), the counterparts of the reference's
 // GenerateUniformBlockedELLIndex, MakeSparseMatrixRandomUniform, IdentityRowSwizzle and
-// SortedRowSwizzle (GEMM/include/bm_test_utils.h:48-128, 197-216 there).  No GPU involved.
+// SortedRowSwizzle (GEMM/include/bm_test_utils.h:48-128, 197-216 there), and of its Host_sddmm
+// (172-194 there).  No GPU involved.
 // Exit status 0 = every expectation held; each failure prints its line.
 #include <cstdio>
 #include <set>
@@ -88,6 +89,24 @@ int main()
             EXPECT(sorted[i] == viaabi[i]);
             if (i > 0) EXPECT(off[sorted[i] + 1] - off[sorted[i]] <= off[sorted[i - 1] + 1] - off[sorted[i - 1]]);
         }
+    }
+    // Host_sddmm: small whole numbers, so that the running fp32 sum equals the integer dot product
+    {
+        const int m_vec = 5, vec = 3, k = 40, n = 7;
+        std::vector<int> li((size_t)m_vec * vec * k), ri((size_t)n * k);
+        std::vector<e4m3> lhs(li.size()), rhs(ri.size());
+        for (size_t t = 0; t < li.size(); ++t) lhs[t] = e4m3((float)(li[t] = (int)(t * 7 % 13) - 6));
+        for (size_t t = 0; t < ri.size(); ++t) rhs[t] = e4m3((float)(ri[t] = (int)(t * 5 % 11) - 5));
+        const std::vector<int> off = {0, 2, 2, 5, 6, 9}, col = {1, 6, 0, 3, 4, 2, 0, 5, 6};
+        std::vector<float> out(col.size() * vec, -1.0f);
+        Host_sddmm<e4m3, float>(m_vec, k, vec, off.data(), col.data(), lhs.data(), rhs.data(), out.data());
+        for (int i = 0; i < m_vec; ++i)
+            for (int j = off[i]; j < off[i + 1]; ++j)
+                for (int v = 0; v < vec; ++v) {
+                    long dot = 0;
+                    for (int l = 0; l < k; ++l) dot += (long)li[((size_t)i * vec + v) * k + l] * ri[(size_t)col[j] * k + l];
+                    EXPECT(out[(size_t)j * vec + v] == (float)dot);
+                }
     }
     if (g_failures == 0) std::printf("all checks passed\n");
     return g_failures == 0 ? 0 : 1;

@@ -171,3 +171,19 @@ def test_sparse_kernel_ids(harness, kernel, shape, env):
     g = re.search(r"([0-9.]+) GFlops on the stored entries", r.stdout)
     assert g and float(g.group(1)) > 0.0
     assert "end BmSparse" in r.stdout
+
+
+@pytest.mark.parametrize("shape,env", [((512, 256, 384), {}), ((96, 1040, 200), {"GEMM_SDDMM_VEC": "16", "GEMM_SPARSE_KEEP": "0.3"}),
+                                       ((60, 100, 50), {"GEMM_SDDMM_VEC": "4"})])
+def test_sddmm_kernel_id(harness, shape, env):
+    """Kernel id 14: the sampled dense-dense product on a pattern from the re-created CSR generator,
+    verified against the harness's Host_sddmm (the reference's host helper of that name,
+    GEMM/include/bm_test_utils.h:172-194 there)."""
+    M, K, N = shape
+    r = harness(M, K, N, 14, 1, 0, 0, env=env)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    assert "sampled e4m3 * e4m3 = fp32" in r.stdout
+    assert "Result Verified!" in r.stdout and "errors." not in r.stdout, r.stdout[-1500:]
+    m = re.search(r"worst \|err\| / tolerance = ([0-9.eE+-]+)", r.stdout)
+    assert m and float(m.group(1)) < 1.0
+    assert "end BmSddmm" in r.stdout

@@ -243,6 +243,42 @@ def test_spmm_csr(pkg, oracle, fs, fb, m, k, n, density, pad):
     assert pkg.lib().fp8gemm_spmm_csr_scratch_bytes(m, k, n) >= m * k
 
 
+@pytest.mark.parametrize("fl,fr", PAIRS)
+@pytest.mark.parametrize("m_vec,vec,k,n,per_row", [(64, 8, 1024, 512, 40), (33, 16, 256, 100, 70), (20, 4, 4096, 64, 17),
+                                                    (7, 1, 144, 30, 5), (5, 16, 8192, 48, 20), (10, 3, 100, 40, 9), (4, 20, 64, 32, 6)])
+def test_sddmm(pkg, oracle, fl, fr, m_vec, vec, k, n, per_row):
+    """Sampled dense-dense product against the oracle's loop (the reference's Host_sddmm): rows with
+    more and fewer than 16 stored entries and empty ones, vector lengths up to 16 on the MFMA,
+    k that is not a whole K step, rows of lhs too long to be held in LDS, and shapes only the
+    one-thread-per-output kernel takes (k % 16 != 0, vec > 16)."""
+    rng = np.random.default_rng(zlib.crc32(repr((fl, fr, m_vec, vec, k, n, per_row)).encode()))
+    lhs = pkg.fill((m_vec * vec, k), fl, seed=0xA11CE + 40 + m_vec, dist="normal", sigma=2.0)
+    rhs = pkg.fill((n, k), fr, seed=0xB0B + 40 + n, dist="normal", sigma=2.0)
+    counts = rng.integers(0, min(n, 2 * per_row) + 1, m_vec)
+    counts[0] = 0
+    offs = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    col = np.concatenate([np.sort(rng.permutation(n)[:c]) for c in counts]).astype(np.int32)
+    out = pkg.sddmm(dev(offs), dev(col), vec, dev(lhs), dev(rhs), l_fmt=fl, r_fmt=fr).cpu().numpy()
+    ref, S = oracle.sddmm(offs, col, vec, lhs, fl, rhs, fr, with_scale=True)
+    tol = oracle.tolerance(k, S) + (2.0 ** -10 * S if k < 1024 else 0.0)
+    check(out, ref, tol)
+
+
+def test_sddmm_small_integers_exact(pkg, oracle):
+    rng = np.random.default_rng(12)
+    m_vec, vec, k, n = 16, 8, 512, 128
+    ints = np.arange(-8, 9, dtype=np.float32)
+    lf, rf = ints[rng.integers(0, 17, (m_vec * vec, k))], ints[rng.integers(0, 17, (n, k))]
+    counts = rng.integers(1, 60, m_vec)
+    offs = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    col = np.concatenate([np.sort(rng.permutation(n)[:c]) for c in counts]).astype(np.int32)
+    out = pkg.sddmm(dev(offs), dev(col), vec, dev(oracle.encode(lf, 0)), dev(oracle.encode(rf, 1)), l_fmt=0, r_fmt=1).cpu().numpy()
+    dense = lf.astype(np.float64) @ rf.astype(np.float64).T
+    for i in range(m_vec):
+        for j in range(offs[i], offs[i + 1]):
+            assert np.array_equal(out[j].astype(np.float64), dense[i * vec:(i + 1) * vec, col[j]])
+
+
 def test_sparse_entry_points_refuse_bad_arguments(pkg):
     import torch
     L = pkg.lib()

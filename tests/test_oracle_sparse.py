@@ -115,3 +115,25 @@ def test_blocked_ell_as_csr_equals_the_dense_loop(oracle, block, ell):
     v, offs, col = oracle.bell_to_csr(vals, bcols, block)
     got = oracle.spmm_csr(v, 0, offs, col, k, B, 0)
     assert np.array_equal(got.view(np.uint32), oracle.gemm_verbatim(dense, 0, B, 0).view(np.uint32))
+
+
+@pytest.mark.parametrize("lfmt,rfmt", [(0, 0), (1, 1), (0, 1), (1, 0)])
+@pytest.mark.parametrize("m_vec,vec,k,n", [(9, 4, 100, 37), (5, 8, 256, 64), (3, 1, 33, 10), (4, 16, 64, 20)])
+def test_sddmm_is_the_dense_product_sampled(oracle, lfmt, rfmt, m_vec, vec, k, n):
+    """Every output of the sampled product is one element of lhs * rhs^T: bit-equal to the dense
+    loop (pinned by tests/test_oracle_gemm.py) gathered at the stored positions, every finite code."""
+    rng = np.random.default_rng(m_vec * 100 + vec + 7 * lfmt + rfmt)
+    lhs = random_codes(rng, (m_vec * vec, k), lfmt)
+    rhs = random_codes(rng, (n, k), rfmt)
+    for a, f in ((lhs, lfmt), (rhs, rfmt)):
+        if f == 1:
+            a[...] = np.where(((a >> 2) & 0x1F) > 24, a & 0x83 | 0x3C, a)
+    counts = rng.integers(0, n, m_vec)
+    offs = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    col = np.concatenate([np.sort(rng.permutation(n)[:c]) for c in counts]).astype(np.int32)
+    got = oracle.sddmm(offs, col, vec, lhs, lfmt, rhs, rfmt)
+    dense = oracle.gemm_verbatim(lhs, lfmt, rhs, rfmt)                  # (m_vec*vec, n)
+    for i in range(m_vec):
+        for j in range(offs[i], offs[i + 1]):
+            want = dense[i * vec:(i + 1) * vec, col[j]]
+            assert np.array_equal(got[j].view(np.uint32), want.view(np.uint32))
