@@ -482,6 +482,8 @@ hipError_t launch_spmv_csr(int m, int k, const uint8_t *values, const int *row_o
     return hipGetLastError();
 }
 
+constexpr int kLdsBytesPerCu = 160 * 1024;
+
 template <int SF, int XF>
 hipError_t launch_spmv_bell(int m, int k, int block, int ell_cols, const uint8_t *values, const int *block_cols,
                             const uint8_t *x, float *y, hipStream_t stream)
@@ -489,15 +491,23 @@ hipError_t launch_spmv_bell(int m, int k, int block, int ell_cols, const uint8_t
     int shift = -1;
     for (int b = 4; b < 31; ++b)
         if (block == (1 << b)) shift = b;
-    // few 16-row groups: two or four waves share the K steps of a group, so that about 2048 waves run
-    const int groups16 = m / 16, steps = (ell_cols * block + 127) / 128;
-    int ksplit = groups16 >= 2048 ? 1 : (groups16 >= 1024 ? 2 : 4);
-    while (ksplit > 1 && steps < 4 * ksplit) ksplit /= 2;
+    const int kell = ell_cols * block;
+    const int lds = (k + 15) / 16 * 16 + kSpmvSumBytes;
+    // R lanes per stored row; a row item = the 64 / R rows a wave has at a time
+    int lanes_per_row = 4;
+    while (lanes_per_row < 64 && lanes_per_row * 16 < kell) lanes_per_row *= 2;
+    const int rows_per_item = 64 / lanes_per_row, items = (m + rows_per_item - 1) / rows_per_item;
+    const int mfma_steps = ((kell + 16 * lanes_per_row - 1) / (16 * lanes_per_row) + 1) / 2;
+    // few items: two or four waves share the MFMA steps of an item, so that about 2048 waves and more run
+    int ksplit = items >= 1024 ? 1 : (items >= 512 ? 2 : 4);
+    while (ksplit > 1 && mfma_steps < 2 * ksplit) ksplit /= 2;
     const int per_wg = 4 / ksplit;
-    int grid = (groups16 + per_wg - 1) / per_wg;
-    if (ksplit == 1 && grid > 512) grid = 512;
-    hipLaunchKernelGGL((spmv_bell_kernel<SF, XF>), dim3((unsigned)grid), dim3(256), (k + 15) / 16 * 16 + 4096, stream, m, k, block,
-                       shift, ell_cols, ksplit, values, block_cols, x, y);
+    int grid = (items + per_wg - 1) / per_wg;
+    // (ksplit 1: no more workgroups than the chip holds at once, eight per CU, fewer where x takes more of the LDS)
+    if (ksplit == 1) grid = std::min(grid, kPlannedCus * std::max(1, std::min(8, kLdsBytesPerCu / lds)));
+    auto kernel = ksplit == 1 ? spmv_bell_kernel<SF, XF, 1> : (ksplit == 2 ? spmv_bell_kernel<SF, XF, 2> : spmv_bell_kernel<SF, XF, 4>);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), lds, stream, m, k, block, shift, ell_cols, lanes_per_row, values,
+                       block_cols, x, y);
     return hipGetLastError();
 }
 

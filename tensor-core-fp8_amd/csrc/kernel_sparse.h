@@ -128,97 +128,126 @@ __global__ __launch_bounds__(64) void spmm_bell_kernel(int m, int k, int n, int 
 }
 
 // Matrix-vector product with S in blocked-ELL form, x (k codes, k <= kSpmvLdsBytes) held in LDS.
-// Bound by reading the stored values once: every wave keeps the loads of DEPTH K steps in flight
-// (the values of a step and the block columns its pieces need) and takes the pieces of x from
-// LDS.  The MFMA multiplies 16 rows of S by 16 copies of x; column 0 is stored.  Lane roles as in
-// spmm_bell_kernel.  Two ways of handing out the work, chosen by the host through `ksplit`:
-//   1: many rows -- the four waves of a workgroup each walk 16-row groups (g, g + waves, ..);
-//   2 or 4: few rows -- that many waves share a group, wave u of them taking K steps u,
-//      u + ksplit, ..; their sums meet in LDS and are added in the order of u.  One pass, the
-//      grid covers every group.
-constexpr int kSpmvLdsBytes = 60 * 1024;       // with the 4 KiB for the sums: the 64 KiB of LDS a kernel gets without asking
+// Bound by reading the stored values once, so the loads take whole lines: one load instruction of a wave
+// takes 1024 contiguous bytes of stored rows (a "slot"), 16 bytes a lane.  (A lane layout that gives each of
+// the MFMA's 16 rows to another row of S, as spmm_bell_kernel has it, loads a quarter of a 128-byte line of
+// each of 16 rows per instruction, and the memory pipeline then carries every line in two requests:
+// measured 24 us against 13.5 us for 59 MB.)  Piece number 4i + q of the slot goes to lane
+// (i = lane % 16, q = lane / 16), so the four lanes that make up row i of the MFMA's first operand hold 64
+// consecutive bytes, and R lanes (a power of two, 4..64; 64 for stored rows of 1024 bytes and more) cover
+// one stored row.  The second operand is, lane for lane, the 16 bytes of x that the lane's piece of S
+// multiplies (from LDS).  The MFMA then computes a 16 x 16 matrix of which only the diagonal is wanted:
+// element (i, i) is the dot product of the 64-byte run i of the slot with its x, and the other 240 are cross
+// terms nobody reads (the matrix unit has the time).  Two slots of the same row feed one MFMA; rows shorter
+// than a slot leave the second half zero.  At a row's end the diagonal is taken out (register i % 4 of lane
+// (i, i / 4)), added over q and over the R / 4 runs of a row, and stored.
+// Two ways of handing out the work, chosen by the host (`ksplit`):
+//   1: a wave handles the 64 / R rows of a "row item" at a time (wave w of all takes items w, w + waves, ..)
+//      and keeps the loads of two MFMA steps in flight across row boundaries (deeper rings measured no
+//      faster: what counts is how many waves are resident, so the host launches as many workgroups as the
+//      chip holds at once);
+//   2 or 4: few rows -- that many waves of a workgroup share an item, wave u of them taking MFMA steps u,
+//      u + ksplit, ..; their sums meet in LDS and are added in the order of u.  One pass: the grid covers
+//      every item.
+constexpr int kSpmvLdsBytes = 60 * 1024;       // with the room for the sums: the 64 KiB of LDS a kernel gets without asking
+constexpr int kSpmvSumBytes = 4 * 16 * 4;      // 16 sums per wave
 
-template <int SF, int XF>
-__global__ __launch_bounds__(256) void spmv_bell_kernel(int m, int k, int block, int block_shift, int ell_cols, int ksplit,
+template <int SF, int XF, int ksplit>
+__global__ __launch_bounds__(256) void spmv_bell_kernel(int m, int k, int block, int block_shift, int ell_cols, int lanes_per_row,
                                                          const uint8_t *__restrict__ values,
                                                          const int *__restrict__ block_cols,
                                                          const uint8_t *__restrict__ x, float *__restrict__ y)
 {
-    constexpr int DEPTH = 8;
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds_x[];      // x, then 4 KiB for the waves' sums
-    const int xbytes = (k + 15) & ~15;
-    bool x_staged = false;
-    // (x is staged in LDS after the first loads of S have been issued, so that their latencies overlap)
-    auto stage_x = [&]() __attribute__((always_inline)) {
-        for (int t = threadIdx.x * 16; t < k; t += 256 * 16) *reinterpret_cast<v4i *>(lds_x + t) = load_piece(x + t);
-        __syncthreads();
-        x_staged = true;
-    };
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_x[];      // x, then kSpmvSumBytes for the waves' sums
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int i = lane & 15, q = lane >> 4;
+    const int lp = 4 * i + q;                                            // the lane's piece of a slot
+    const int R = lanes_per_row, rows_per_item = 64 / R, G = R / 4;      // G: 64-byte runs per row and slot
     const int kell = ell_cols * block;
-    const int steps = (kell + 127) / 128;
-    const int groups = m / 16;
+    const int U = (kell + 16 * R - 1) / (16 * R);                        // slots per row (1 when R < 64)
+    const int NM = (U + 1) / 2;                                          // MFMA steps per row item
+    const int items = (m + rows_per_item - 1) / rows_per_item;
+    const int sub = wave % ksplit;                                       // which share of an item's MFMA steps
+    const int per_wg = 4 / ksplit;                                       // items a workgroup has at a time
+    const int waves = gridDim.x * per_wg, w = blockIdx.x * per_wg + wave / ksplit;
+    const int mine = w < items ? (items - w + waves - 1) / waves : 0;    // row items of this wave (ksplit > 1: at most 1)
+    const int share = NM > sub ? (NM - sub + ksplit - 1) / ksplit : 0;   // MFMA steps sub, sub + ksplit, .. of an item
+    const int total = mine * share;                                      // MFMA steps of this wave
+    const int per_item = share > 0 ? share : 1;
+    const int sub_row = lp / R, in_row = lp - sub_row * R;
     const v4i zero = {0, 0, 0, 0};
-    const int sub = wave % ksplit;                                      // which share of the K steps
-    const int per_wg = 4 / ksplit;                                      // groups a workgroup has at a time
-    const int stride = ksplit == 1 ? gridDim.x * 4 : groups;            // (ksplit > 1: a single pass)
-    for (int g = blockIdx.x * per_wg + wave / ksplit; g < groups || ksplit > 1; g += stride) {
-        const bool have = g < groups;
-        v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
-        const int row0 = have ? g * 16 : 0;
-        if (have) {
-            const int *cols = block_cols + (size_t)(row0 / block) * ell_cols;
-            const uint8_t *srow = values + (size_t)(row0 + i) * kell;
-            const int mine = (steps - sub + ksplit - 1) / ksplit;       // K steps sub, sub + ksplit, ..
-            v4i a[DEPTH][2];
-            int at[DEPTH][2];      // where in x the piece lies; -1: nowhere (padding block, or past the stored row)
-            auto fetch = [&](int u, int d) __attribute__((always_inline)) {
+
+    struct Step {
+        v4i s[2];
+        int at[2];      // where in x the piece lies; -1: nowhere (padding block, past the stored row or the last row)
+    };
+    // step t of this wave: row item w + (t / share) * waves, MFMA step sub + (t % share) * ksplit of it,
+    // which takes slots 2 * step and the one after
+    auto fetch = [&](int t, Step &f) __attribute__((always_inline)) {
+        const int it = t / per_item, ms = sub + (t - it * per_item) * ksplit;
+        const int row = (w + it * waves) * rows_per_item + sub_row;
 #pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const int p = (sub + u * ksplit) * 128 + (2 * q + h) * 16;
-                    a[d][h] = zero;
-                    at[d][h] = -1;
-                    if (p < kell) {
-                        const int blk = block_shift >= 0 ? p >> block_shift : p / block;
-                        const int c = cols[blk];
-                        a[d][h] = load_piece(srow + p);
-                        at[d][h] = c < 0 ? -1 : c * block + (p - blk * block);
-                    }
-                }
-            };
-#pragma unroll
-            for (int d = 0; d < DEPTH; ++d)
-                if (d < mine) fetch(d, d);
-            if (!x_staged) stage_x();                                  // (uniform over the workgroup: first pass of every wave)
-            for (int u0 = 0; u0 < mine; u0 += DEPTH) {
-#pragma unroll
-                for (int d = 0; d < DEPTH; ++d) {
-                    if (u0 + d < mine) {                               // (uniform)
-                        v4i xp[2];
-#pragma unroll
-                        for (int h = 0; h < 2; ++h) xp[h] = at[d][h] >= 0 ? *reinterpret_cast<const v4i *>(lds_x + at[d][h]) : zero;
-                        acc = mfma_16x16x128<SF, XF>(pack8(a[d][0], a[d][1]), pack8(xp[0], xp[1]), acc);
-                        if (u0 + d + DEPTH < mine) fetch(u0 + d + DEPTH, d);
-                    }
-                }
+        for (int h = 0; h < 2; ++h) {
+            const int u = 2 * ms + h;
+            const int p = (u * R + in_row) * 16;
+            f.s[h] = zero;
+            f.at[h] = -1;
+            if (t < total && u < U && row < m && p < kell) {
+                const int blk = block_shift >= 0 ? p >> block_shift : p / block;
+                const int c = block_cols[(size_t)(row / block) * ell_cols + blk];
+                f.s[h] = __builtin_nontemporal_load(reinterpret_cast<const v4i *>(values + (size_t)row * kell + p));
+                f.at[h] = c < 0 ? -1 : c * block + (p - blk * block);
             }
         }
-        if (!x_staged) stage_x();                                      // a wave without a group still joins the barrier
-        if (ksplit > 1) {
-            v4f *sums = reinterpret_cast<v4f *>(lds_x + xbytes);
-            sums[wave * 64 + lane] = acc;
-            __syncthreads();
-            if (sub == 0)
-                for (int u = 1; u < ksplit; ++u) acc += sums[(wave + u) * 64 + lane];
-        }
-        if (have && sub == 0 && i == 0) {
+    };
+    Step ring[2];
+    fetch(0, ring[0]);
+    // (x is staged after the first loads of S have been issued, so that their latencies overlap)
+    for (int t = threadIdx.x * 16; t < k; t += 256 * 16) *reinterpret_cast<v4i *>(lds_x + t) = load_piece(x + t);
+    __syncthreads();
+
+    v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    float part = 0.0f;                                                   // ksplit > 1: this wave's share of its item's sums
+    auto consume = [&](int t, const Step &f) __attribute__((always_inline)) {
+        if (t >= total) return;                                          // (uniform)
+        v4i xs[2];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) y[row0 + 4 * q + r] = acc[r];
+        for (int h = 0; h < 2; ++h) xs[h] = f.at[h] >= 0 ? *reinterpret_cast<const v4i *>(lds_x + f.at[h]) : zero;
+        acc = mfma_16x16x128<SF, XF>(pack8(f.s[0], f.s[1]), pack8(xs[0], xs[1]), acc);
+        const int it = t / per_item;
+        if (t - it * per_item == share - 1) {                            // (uniform) this wave's part of the item is complete
+            const int r = i & 3;
+            float v = r == 0 ? acc[0] : (r == 1 ? acc[1] : (r == 2 ? acc[2] : acc[3]));
+            v = (i >> 2) == q ? v : 0.0f;
+            v += __shfl_xor(v, 16, 64);
+            v += __shfl_xor(v, 32, 64);
+            for (int off = 1; off < G; off <<= 1) v += __shfl_xor(v, off, 64);
+            const int row = (w + it * waves) * rows_per_item + i / G;
+            if (ksplit == 1) {
+                if (q == 0 && i % G == 0 && row < m) y[row] = v;
+            } else {
+                part = v;
+            }
+            acc = v4f{0.0f, 0.0f, 0.0f, 0.0f};
         }
-        if (ksplit > 1) break;
+    };
+    for (int t0 = 0; t0 < total; t0 += 2) {
+        fetch(t0 + 1, ring[1]);
+        consume(t0, ring[0]);
+        fetch(t0 + 2, ring[0]);
+        consume(t0 + 1, ring[1]);
     }
-    if (!x_staged) stage_x();          // a wave that had no group at all: every wave passes the barrier exactly once
+    if (ksplit > 1) {                                                    // (uniform over the grid)
+        float *sums = reinterpret_cast<float *>(lds_x + ((k + 15) & ~15));
+        if (q == 0) sums[wave * 16 + i] = part;
+        __syncthreads();
+        const int row = w * rows_per_item + i / G;
+        if (sub == 0 && q == 0 && i % G == 0 && w < items && row < m) {
+            float v = part;
+            for (int u = 1; u < ksplit; ++u) v += sums[(wave + u) * 16 + i];
+            y[row] = v;
+        }
+    }
 }
 
 // y[row] = sum over the stored entries of the row of float(values[e]) * float(x[col[e]]):
