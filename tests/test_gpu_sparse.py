@@ -264,6 +264,33 @@ def test_sddmm(pkg, oracle, fl, fr, m_vec, vec, k, n, per_row):
     check(out, ref, tol)
 
 
+def test_sddmm_at_benchmark_size_is_the_dense_product_sampled(pkg):
+    """The benchmark's shape (8192 x 8192 outputs in vectors of 8, one in ten stored, K = 512), too large
+    for the CPU loop: every stored output is an element of lhs * rhs^T, which the library's dense GEMM
+    (held to the oracle by its own tests) computes in another order; the bound's sum of magnitudes comes
+    from the same GEMM on the operands with their sign bits cleared."""
+    import torch
+    m_vec, vec, n, k = 1024, 8, 8192, 512
+    rng = np.random.default_rng(77)
+    mask = rng.random((m_vec, n)) < 0.10
+    offs = np.concatenate([[0], np.cumsum(mask.sum(axis=1))]).astype(np.int32)
+    rows, col = np.nonzero(mask)
+    lhs = dev(pkg.fill((m_vec * vec, k), 0, seed=0xA11CE + 77, dist="normal"))
+    rhs = dev(pkg.fill((n, k), 0, seed=0xB0B + 77, dist="normal"))
+    out = pkg.sddmm(dev(offs), dev(col.astype(np.int32)), vec, lhs, rhs, l_fmt=0, r_fmt=0)
+    dense = pkg.gemm(lhs, rhs, a_fmt=0, b_fmt=0)
+    mags = pkg.gemm(lhs & 0x7F, rhs & 0x7F, a_fmt=0, b_fmt=0)
+    torch.cuda.synchronize()
+    r = torch.from_numpy(rows).to("cuda")[:, None] * vec + torch.arange(vec, device="cuda")[None, :]
+    c = torch.from_numpy(col).to("cuda")[:, None].expand(-1, vec)
+    want, S = dense[r, c], mags[r, c]
+    assert out.shape == want.shape
+    # both sides are reordered fp32 sums of the same exact products (each within the bound of the running sum)
+    tol = 2.0 * (2.0 * k * 2.0 ** -24 + 2.0 ** -10) * S
+    assert bool((torch.abs(out - want) <= tol).all())
+    assert float(torch.abs(out).max()) > 0.0
+
+
 def test_sddmm_small_integers_exact(pkg, oracle):
     rng = np.random.default_rng(12)
     m_vec, vec, k, n = 16, 8, 512, 128
@@ -294,4 +321,13 @@ def test_sparse_entry_points_refuse_bad_arguments(pkg):
     assert L.fp8gemm_spmm_bell(64, 64, 16, 16, 4, v.data_ptr(), 2, c.data_ptr(), b.data_ptr(), 0, o.data_ptr(), None) == 1
     assert L.fp8gemm_spmv_csr(0, 64, v.data_ptr(), 0, c.data_ptr(), c.data_ptr(), None, b.data_ptr(), 0, o.data_ptr(), None) == 1
     assert L.fp8gemm_spmm_csr(4, 64, 16, v.data_ptr(), 0, None, c.data_ptr(), b.data_ptr(), 0, o.data_ptr(), None) == 1
+    # sampled product: a pattern with no stored entry at all is a launch that writes nothing
+    offs = torch.zeros(5, dtype=torch.int32, device="cuda")
+    o.fill_(7.0)
+    assert L.fp8gemm_sddmm(4, 64, 16, offs.data_ptr(), c.data_ptr(), v.data_ptr(), 0, b.data_ptr(), 0, o.data_ptr(), None) == 0
+    assert L.fp8gemm_sddmm(0, 64, 16, offs.data_ptr(), c.data_ptr(), v.data_ptr(), 0, b.data_ptr(), 0, o.data_ptr(), None) == 1
+    assert L.fp8gemm_sddmm(4, 64, 0, offs.data_ptr(), c.data_ptr(), v.data_ptr(), 0, b.data_ptr(), 0, o.data_ptr(), None) == 1
+    assert L.fp8gemm_sddmm(4, 64, 16, None, c.data_ptr(), v.data_ptr(), 0, b.data_ptr(), 0, o.data_ptr(), None) == 1
+    assert L.fp8gemm_sddmm(4, 64, 16, offs.data_ptr(), c.data_ptr(), v.data_ptr(), 3, b.data_ptr(), 0, o.data_ptr(), None) == 1
     torch.cuda.synchronize()
+    assert bool((o == 7.0).all())
