@@ -36,7 +36,7 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E peak, GB/s
 # HBM-side bytes moved by one 8192^3 launch of the tiled kernel: a constant taken from the
 # rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs summarised under profiles/ (each scaled by
 # what the same counter reads for a plain copy kernel of known size), not a reading of this run.
-TRAFFIC_8192 = {"fetch_kib": 393439, "fetch_scale": 2.0, "write_kib": 262607, "write_scale": 1.0}
+TRAFFIC_8192 = {"fetch_kib": 393431, "fetch_scale": 2.0, "write_kib": 262624, "write_scale": 1.0}
 TRAFFIC_BYTES_8192 = int((TRAFFIC_8192["fetch_kib"] * TRAFFIC_8192["fetch_scale"] +
                           TRAFFIC_8192["write_kib"] * TRAFFIC_8192["write_scale"]) * 1024)
 
