@@ -210,7 +210,7 @@ def main():
         return go
 
     def time_settled(m, k, n, fa, fb, A_host, B_host, steps, rows):
-        """One more BASELINE shape through fp8gemm_launch: operands to HBM, clocks settled under
+        """One more benchmark shape through fp8gemm_launch: operands to HBM, clocks settled under
         this shape's own load, `steps` timed launches, a sample of full rows against the CPU
         oracle (checker only).  Returns the record for the JSON line."""
         dA = torch.from_numpy(A_host).to(dev)
@@ -302,7 +302,7 @@ def main():
     del A, B, C
     torch.cuda.empty_cache()
 
-    # ---------------------------------------------------------------- the other compute-bound BASELINE shapes
+    # ---------------------------------------------------------------- the other compute-bound benchmark shapes
     # (each through fp8gemm_launch, clocks settled under its own load; `value` stays the 8192^3 figure)
     square_sweep = [{"M": M, "N": N, "K": K, "a": "e4m3", "b": "e4m3", "steps": args.steps, "ms": ms, "tflops": tflops,
                      "frac_of_fp8_peak": tflops / PEAK_FP8_TFLOPS, "plan": list(pkg.plan(M, K, N)), "parity": parity}]
