@@ -156,8 +156,16 @@ def test_spmm_bell_one_hot_is_bit_exact(pkg, oracle, fs, fb):
 
 
 @pytest.mark.parametrize("fs,fx", PAIRS)
-@pytest.mark.parametrize("block,ell,m,k", [(16, 8, 1024, 2048), (128, 4, 512, 4096), (32, 1, 64, 64)])
+@pytest.mark.parametrize("block,ell,m,k", [(16, 8, 1024, 2048), (128, 4, 512, 4096), (32, 1, 64, 64),
+                                           (64, 112, 256, 8192),        # stored rows of 7 slots of 1 KiB (an odd count), two waves to a row
+                                           (64, 256, 64, 16384),        # few long rows: four waves to a row
+                                           (64, 24, 2048, 4096),        # a slot and a half per row, several rows per wave
+                                           (48, 5, 960, 960),           # blocks that are no power of two, 16 lanes to a row
+                                           (16, 3, 4096, 1024),         # rows shorter than the four lanes they get
+                                           (256, 8, 16384, 4096)])      # more row items than resident waves
 def test_spmv_bell(pkg, oracle, fs, fx, block, ell, m, k):
+    """Row lengths on every side of the kernel's slot of 1024 bytes, row counts that choose each of its
+    ways of sharing the work, padding blocks."""
     rng = np.random.default_rng(zlib.crc32(repr((fs, fx, block, ell, m, k)).encode()))
     vals, bcols = random_bell(rng, m, k, block, ell, fs, pad_some=True, encode=oracle.encode, sigma=2.0)
     x = pkg.fill((k,), fx, seed=0xA11CE + 80 + block, dist="normal", sigma=2.0)
