@@ -517,15 +517,17 @@ hipError_t launch_sddmm(int m_vec, int k, int vec, const int *row_offsets, const
 {
     const bool fast = vec <= 16 && k % 16 == 0 && (reinterpret_cast<uintptr_t>(lhs) | reinterpret_cast<uintptr_t>(rhs)) % 16 == 0;
     const size_t lds = (size_t)vec * (k + kSddmmLdsPad);
-    if (fast && lds <= (size_t)kSddmmLdsBytes)
-        hipLaunchKernelGGL((sddmm_kernel<LF, RF, true>), dim3((unsigned)m_vec), dim3(256), lds, stream, k, vec, row_offsets, col, lhs,
+    const bool alds = lds <= (size_t)kSddmmLdsBytes;
+    const bool wide = vec % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    if (fast) {
+        auto kernel = alds ? (wide ? sddmm_kernel<LF, RF, true, true> : sddmm_kernel<LF, RF, true, false>)
+                           : (wide ? sddmm_kernel<LF, RF, false, true> : sddmm_kernel<LF, RF, false, false>);
+        hipLaunchKernelGGL(kernel, dim3((unsigned)m_vec), dim3(64 * kSddmmWaves), alds ? lds : 0, stream, k, vec, row_offsets, col, lhs,
                            rhs, out);
-    else if (fast)
-        hipLaunchKernelGGL((sddmm_kernel<LF, RF, false>), dim3((unsigned)m_vec), dim3(256), 0, stream, k, vec, row_offsets, col, lhs,
-                           rhs, out);
-    else
+    } else {
         hipLaunchKernelGGL((sddmm_general_kernel<LF, RF>), dim3((unsigned)m_vec), dim3(256), 0, stream, m_vec, k, vec, row_offsets, col,
                            lhs, rhs, out);
+    }
     return hipGetLastError();
 }
 

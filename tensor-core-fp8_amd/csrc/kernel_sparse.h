@@ -428,23 +428,28 @@ __global__ __launch_bounds__(256) void csr_densify_rows_kernel(int m, int k, con
 // Sampled dense-dense product with a vector-sparse output pattern (the reference's Host_sddmm,
 // GEMM/include/bm_test_utils.h:172-194): out[j * vec + v] = lhs[i * vec + v] . rhs[col[j]] for every
 // stored entry j of vector row i; lhs (m_vec * vec) x k and rhs n x k, both row-major: every dot
-// product runs along K on both sides, which is the MFMA's operand layout.  One workgroup of four waves per
-// vector row; a wave takes 16 stored entries at a time (wave, wave + 4, ..): the up to 16 rows of lhs are the
-// MFMA's A, the 16 gathered rows of rhs its B, and out[j][v] is element (v, j) of the 16 x 16 result.
-// Lane (i = lane % 16, q = lane / 16) supplies 32 bytes of row i per K step; the next step's loads are
-// issued before the current MFMA.  The gathered rows of rhs come out of cache at whatever rate the CU can
-// keep loads in flight, so the rows of lhs, which every chunk of the vector row needs again, are taken from
-// LDS instead when they fit (ALDS: rows kSddmmLdsPad bytes apart from a multiple of 128, so that the 16 lanes
-// of a quarter read 16 different bank groups); otherwise they are loaded next to the rows of rhs.
+// product runs along K on both sides, which is the MFMA's operand layout.  One workgroup of eight waves per
+// vector row; a wave takes 16 stored entries at a time (chunks wave, wave + 8, ..): the up to 16 rows of lhs
+// are the MFMA's A, the 16 gathered rows of rhs its B, and out[j][v] is element (v, j) of the 16 x 16 result.
+// Lane (i = lane % 16, q = lane / 16) supplies 32 bytes of row i per K step.  What bounds the kernel is the
+// latency of the gather -- the column index first, then the row of rhs it names -- so both run ahead of the
+// MFMA across chunk boundaries: the column indices two chunks ahead, the rows of rhs one K step ahead (the
+// last K step of a chunk fetches the first of the next), and eight waves to a row keep 32 waves on a CU.
+// (With everything fetched inside the chunk that used it: 24.4 us for 840 k stored vectors at K = 128; now 11.)
+// The rows of lhs, which every chunk of the vector row needs again, are taken from LDS when they fit (ALDS:
+// rows kSddmmLdsPad bytes apart from a multiple of 128, so that the 16 lanes of a quarter read 16 different
+// bank groups); otherwise they are loaded next to the rows of rhs.  WIDE: vec % 4 == 0 and out 16-byte
+// aligned, a lane's four results leave in one store.
 // Requirements checked by the host: vec <= 16, k % 16 == 0, 16-byte aligned lhs and rhs; ALDS:
-// 16 * (k + kSddmmLdsPad) bytes of dynamic LDS.
+// vec * (k + kSddmmLdsPad) bytes of dynamic LDS.
 constexpr int kSddmmLdsPad = 16;
 constexpr int kSddmmLdsBytes = 64 * 1024;
+constexpr int kSddmmWaves = 8;
 
-template <int LF, int RF, bool ALDS>
-__global__ __launch_bounds__(256) void sddmm_kernel(int k, int vec, const int *__restrict__ row_offsets,
-                                                     const int *__restrict__ col, const uint8_t *__restrict__ lhs,
-                                                     const uint8_t *__restrict__ rhs, float *__restrict__ out)
+template <int LF, int RF, bool ALDS, bool WIDE>
+__global__ __launch_bounds__(64 * kSddmmWaves) void sddmm_kernel(int k, int vec, const int *__restrict__ row_offsets,
+                                                                  const int *__restrict__ col, const uint8_t *__restrict__ lhs,
+                                                                  const uint8_t *__restrict__ rhs, float *__restrict__ out)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t sddmm_lds[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -458,34 +463,50 @@ __global__ __launch_bounds__(256) void sddmm_kernel(int k, int vec, const int *_
     const int ai = i < vec ? i : vec - 1;
     const uint8_t *arow = lhs + (size_t)(vrow * vec + ai) * k;
     const int lds_stride = k + kSddmmLdsPad;
+    // the entry this lane gathers for chunk number c of this wave (past the row's end: its last entry again)
+    auto entry_of = [&](int c) __attribute__((always_inline)) {
+        const long j = (long)e0 + ((long)wave + (long)kSddmmWaves * c) * 16 + i;
+        return j < e1 ? (int)j : e1 - 1;
+    };
+    const int chunks = (e1 - e0 + 15) / 16;
+    const int mine = chunks > wave ? (chunks - wave + kSddmmWaves - 1) / kSddmmWaves : 0;      // chunks of this wave
+    int col_next = 0, col_after = 0;
+    const uint8_t *brow = rhs;
+    if (mine > 0) {
+        brow = rhs + (size_t)col[entry_of(0)] * k;
+        col_next = col[entry_of(1)];
+    }
+    struct Step {
+        v4i a[2], b[2];
+    };
+    auto fetch = [&](const uint8_t *b_row, int s, Step &f) __attribute__((always_inline)) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int p = s * 128 + (2 * q + h) * 16;
+            if constexpr (!ALDS) f.a[h] = p < k ? load_piece(arow + p) : zero;
+            f.b[h] = p < k ? load_piece(b_row + p) : zero;
+        }
+    };
+    Step cur, nxt;
+    if (mine > 0) fetch(brow, 0, cur);
     if constexpr (ALDS) {
         const int per_row = k / 16;
-        for (int t = threadIdx.x; t < vec * per_row; t += 256) {
+        for (int t = threadIdx.x; t < vec * per_row; t += 64 * kSddmmWaves) {
             const int r = t / per_row, c = t - r * per_row;
             *reinterpret_cast<v4i *>(sddmm_lds + r * lds_stride + c * 16) = load_piece(lhs + (size_t)(vrow * vec + r) * k + c * 16);
         }
         __syncthreads();
     }
     const uint8_t *alds = sddmm_lds + ai * lds_stride;
-    for (int j0 = e0 + wave * 16; j0 < e1; j0 += 64) {
-        const int j = j0 + i < e1 ? j0 + i : e1 - 1;          // (entries past the row's end re-read its last one)
-        const uint8_t *brow = rhs + (size_t)col[j] * k;
-        struct Step {
-            v4i a[2], b[2];
-        };
-        auto fetch = [&](int s, Step &f) __attribute__((always_inline)) {
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const int p = s * 128 + (2 * q + h) * 16;
-                if constexpr (!ALDS) f.a[h] = p < k ? load_piece(arow + p) : zero;
-                f.b[h] = p < k ? load_piece(brow + p) : zero;
-            }
-        };
+    for (int c = 0; c < mine; ++c) {
+        col_after = col[entry_of(c + 2)];
+        const uint8_t *brow_next = rhs + (size_t)col_next * k;
         v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
-        Step cur, nxt;
-        fetch(0, cur);
         for (int s = 0; s < steps; ++s) {
-            if (s + 1 < steps) fetch(s + 1, nxt);
+            if (s + 1 < steps)
+                fetch(brow, s + 1, nxt);
+            else
+                fetch(brow_next, 0, nxt);                     // (after the last chunk: the last entry's row once more)
             if constexpr (ALDS) {
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
@@ -496,12 +517,19 @@ __global__ __launch_bounds__(256) void sddmm_kernel(int k, int vec, const int *_
             acc = mfma_16x16x128<LF, RF>(pack8(cur.a[0], cur.a[1]), pack8(cur.b[0], cur.b[1]), acc);
             cur = nxt;
         }
-        // register r of lane (i, q) holds lhs row 4q + r times rhs row col[j0 + i]
-        if (j0 + i < e1) {
+        // register r of lane (i, q) holds lhs row 4q + r times rhs row col[j]
+        const long j = (long)e0 + ((long)wave + (long)kSddmmWaves * c) * 16 + i;
+        if (j < e1) {
+            if constexpr (WIDE) {
+                if (4 * q < vec) *reinterpret_cast<v4f *>(out + (size_t)j * vec + 4 * q) = acc;
+            } else {
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-                if (4 * q + r < vec) out[(size_t)(j0 + i) * vec + 4 * q + r] = acc[r];
+                for (int r = 0; r < 4; ++r)
+                    if (4 * q + r < vec) out[(size_t)j * vec + 4 * q + r] = acc[r];
+            }
         }
+        brow = brow_next;
+        col_next = col_after;
     }
 }
 
