@@ -314,6 +314,79 @@ def test_sddmm_small_integers_exact(pkg, oracle):
             assert np.array_equal(out[j].astype(np.float64), dense[i * vec:(i + 1) * vec, col[j]])
 
 
+def _bell_on_device(pkg, m, k, block, ell, seed):
+    """A blocked-ELL operand of normal values, and the dense matrix its blocks spell out, both on the device."""
+    import torch
+    rng = np.random.default_rng(seed)
+    nbr, nbc = m // block, k // block
+    bcols = np.stack([np.sort(rng.permutation(nbc)[:ell]) for _ in range(nbr)]).astype(np.int32)
+    vals = dev(pkg.fill((m, ell * block), 0, seed=0xA11CE + seed, dist="normal"))
+    dense = torch.zeros((nbr, block, nbc, block), dtype=torch.uint8, device="cuda")
+    rows = torch.arange(nbr, device="cuda")[:, None].expand(-1, ell)
+    dense[rows, :, dev(bcols).long(), :] = vals.view(nbr, block, ell, block).permute(0, 2, 1, 3)
+    return vals, bcols, dense.view(m, k)
+
+
+def _within_reordering(out, want, mags, terms):
+    """Two fp32 sums of the same exact products in different orders, `mags` the sum of their magnitudes."""
+    import torch
+    tol = 2.0 * (2.0 * terms * 2.0 ** -24 + 2.0 ** -10) * mags
+    assert bool(torch.isfinite(out).all()) and bool((torch.abs(out - want) <= tol).all())
+    assert float(torch.abs(out).max()) > 0.0
+
+
+@pytest.mark.parametrize("m,k,n,block,ell", [(8192, 8192, 8192, 256, 8), (8192, 8192, 8192, 128, 16), (4096, 4096, 4096, 32, 32)])
+def test_spmm_bell_at_benchmark_size_is_the_dense_gemm_on_the_blocks_spelled_out(pkg, m, k, n, block, ell):
+    """The benchmark's blocked-ELL shapes, too large for the CPU loop: zeros add nothing, so the product
+    equals the library's dense GEMM (held to the oracle by its own tests) on the dense matrix the stored
+    blocks spell out, up to the order of the sum; the sum of magnitudes for the bound comes from the same
+    GEMM on the operands with their sign bits cleared."""
+    import torch
+    vals, bcols, dense = _bell_on_device(pkg, m, k, block, ell, seed=block)
+    B = dev(pkg.fill((n, k), 0, seed=0xB0B + block, dist="normal"))
+    out = pkg.spmm_bell(vals, dev(bcols), block, B, k, s_fmt=0, b_fmt=0)
+    want = pkg.gemm(dense, B, a_fmt=0, b_fmt=0)
+    mags = pkg.gemm(dense & 0x7F, B & 0x7F, a_fmt=0, b_fmt=0)
+    torch.cuda.synchronize()
+    _within_reordering(out, want, mags, ell * block)
+
+
+def test_spmv_at_benchmark_size_is_the_dense_matrix_vector_product(pkg):
+    """The benchmark's two matrix-vector shapes (28672 x 8192: a quarter of the 64 x 64 blocks, and one
+    element in ten in CSR) against the library's dense GEMV on the matrix the operand spells out."""
+    import torch
+    m, k = 28672, 8192
+    x = dev(pkg.fill((k,), 0, seed=0x5BA, dist="normal"))
+    L = pkg.lib()
+
+    def gemv(w):
+        y = torch.empty(m, dtype=torch.float32, device="cuda")
+        pkg.check(L.fp8gemm_gemv(m, k, w.data_ptr(), 0, x.data_ptr(), 0, y.data_ptr(), None))
+        return y
+    vals, bcols, dense = _bell_on_device(pkg, m, k, 64, 32, seed=5)
+    y = pkg.spmm_bell(vals, dev(bcols), 64, x, k, s_fmt=0, b_fmt=0)
+    want = gemv(dense)
+    magx = torch.empty_like(want)                          # sum of |a| * |x|: the same GEMV with the sign bits cleared
+    xa = x & 0x7F
+    pkg.check(L.fp8gemm_gemv(m, k, (dense & 0x7F).data_ptr(), 0, xa.data_ptr(), 0, magx.data_ptr(), None))
+    torch.cuda.synchronize()
+    _within_reordering(y, want, magx, 32 * 64)
+    del vals, dense
+    # CSR: one element in ten
+    rng = np.random.default_rng(9)
+    mask = torch.from_numpy(rng.random((m, k)) < 0.10).cuda()
+    codes = dev(pkg.fill((m, k), 0, seed=0xA11CE + 9, dist="normal"))
+    dense = torch.where(mask, codes, torch.zeros_like(codes))
+    offs = torch.zeros(m + 1, dtype=torch.int32, device="cuda")
+    offs[1:] = torch.cumsum(mask.sum(dim=1), 0).to(torch.int32)
+    col = torch.nonzero(mask)[:, 1].to(torch.int32).contiguous()
+    y = pkg.spmm_csr(codes[mask].contiguous(), offs, col, x, k, s_fmt=0, b_fmt=0)
+    want = gemv(dense)
+    pkg.check(L.fp8gemm_gemv(m, k, (dense & 0x7F).data_ptr(), 0, xa.data_ptr(), 0, magx.data_ptr(), None))
+    torch.cuda.synchronize()
+    _within_reordering(y, want, magx, 8192)
+
+
 def test_sparse_entry_points_refuse_bad_arguments(pkg):
     import torch
     L = pkg.lib()
