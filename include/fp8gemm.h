@@ -82,7 +82,10 @@ int fp8gemm_gemv(int n, int k, const void *w, int w_fmt, const void *x, int x_fm
  * (GEMM/include/bm_test_utils.h:48-68 blocked-ELL column lists, :71-128 compressed sparse rows
  * with optional row padding, :197-216 row orders).  Every stored entry contributes
  * float(value) * float(b[j][column]) to out[i][j], fp32 accumulation; all pointers are device
- * pointers; formats as for the GEMM; launches are asynchronous on `stream`.
+ * pointers; formats as for the GEMM; launches are asynchronous on `stream`.  The matrix-vector
+ * products and fp8gemm_sddmm allocate nothing; fp8gemm_spmm_bell and fp8gemm_spmm_csr take scratch
+ * from the stream's pool like fp8gemm_launch (so a call that is captured into a HIP graph must have
+ * been made once on that stream before).
  *
  * Blocked-ELL: square blocks of `block` x `block` elements (block % 16 == 0, m % block == 0,
  * k % block == 0); every block row stores ell_cols blocks.  values: m x (ell_cols * block)

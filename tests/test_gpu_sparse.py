@@ -387,6 +387,63 @@ def test_spmv_at_benchmark_size_is_the_dense_matrix_vector_product(pkg):
     _within_reordering(y, want, magx, 8192)
 
 
+def test_sparse_launches_replay_in_a_hip_graph(pkg):
+    """The matrix-vector products and the sampled product allocate nothing and clear nothing, and the blocked-ELL
+    SpMM takes its scratch from the stream's pool, which a first eager call has sized: all four captured into
+    one HIP graph and replayed on new operand values, with eager work between the replays, give the eager
+    results bit for bit."""
+    import torch
+    rng = np.random.default_rng(4)
+    m, k, n, block, ell = 2048, 4096, 512, 64, 8
+    vals, bcols, _ = _bell_on_device(pkg, m, k, block, ell, seed=21)
+    bc = dev(bcols)
+    B = dev(pkg.fill((n, k), 0, seed=0xB0B + 21, dist="normal"))
+    x = dev(pkg.fill((k,), 0, seed=0xB0B + 22, dist="normal"))
+    mask = rng.random((m, k)) < 0.05
+    offs = dev(np.concatenate([[0], np.cumsum(mask.sum(axis=1))]).astype(np.int32))
+    col = dev(np.nonzero(mask)[1].astype(np.int32))
+    cv = dev(pkg.fill((int(mask.sum()),), 0, seed=0xA11CE + 23, dist="normal"))
+    vmask = rng.random((m // 8, n)) < 0.2
+    voffs = dev(np.concatenate([[0], np.cumsum(vmask.sum(axis=1))]).astype(np.int32))
+    vcol = dev(np.nonzero(vmask)[1].astype(np.int32))
+    lhs = dev(pkg.fill((m, 256), 0, seed=0xA11CE + 24, dist="normal"))
+    rhs = dev(pkg.fill((n, 256), 0, seed=0xB0B + 24, dist="normal"))
+    outs = [torch.empty((m, n), dtype=torch.float32, device="cuda"), torch.empty(m, dtype=torch.float32, device="cuda"),
+            torch.empty(m, dtype=torch.float32, device="cuda"), torch.empty((int(vmask.sum()), 8), dtype=torch.float32, device="cuda")]
+
+    def launches(stream):
+        pkg.spmm_bell(vals, bc, block, B, k, s_fmt=0, b_fmt=0, out=outs[0], stream=stream)
+        pkg.spmm_bell(vals, bc, block, x, k, s_fmt=0, b_fmt=0, out=outs[1], stream=stream)
+        pkg.spmm_csr(cv, offs, col, x, k, s_fmt=0, b_fmt=0, out=outs[2], stream=stream)
+        pkg.sddmm(voffs, vcol, 8, lhs, rhs, l_fmt=0, r_fmt=0, out=outs[3], stream=stream)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launches(side)                                   # (sizes the stream's scratch pool before the capture)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        launches(side)
+    for rep in range(3):
+        # new operand values in place, then eager work of the program's own, then the replay
+        new = dev(pkg.fill((m, ell * block), 0, seed=0xA11CE + 30 + rep, dist="normal"))
+        vals.copy_(new)
+        x.copy_(dev(pkg.fill((k,), 0, seed=0xB0B + 30 + rep, dist="normal")))
+        lhs.copy_(dev(pkg.fill((m, 256), 0, seed=0xA11CE + 40 + rep, dist="normal")))
+        torch.cuda.synchronize()
+        for o in outs:
+            o.fill_(-1.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs]
+        launches(None)
+        torch.cuda.synchronize()
+        for g, o in zip(got, outs):
+            assert torch.equal(g, o)
+    assert float(torch.abs(outs[0]).max()) > 0.0
+
+
 def test_sparse_entry_points_refuse_bad_arguments(pkg):
     import torch
     L = pkg.lib()
